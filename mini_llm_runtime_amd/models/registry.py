@@ -1,6 +1,7 @@
 """One registry from an architecture's name to its configuration class and its
-builder.  `config.json["architectures"][0]` is the key, as everywhere in the
-framework; a config without that key is looked up by its `model_type`.
+builder.  `config.json["architectures"][0]` (or the string under `architecture`) is the
+key, as everywhere in the framework; a config without either is looked up by
+its `model_type`.
 
 The reference has no registry: its model type gate is an `if`
 (src/mini_llm_runtime/qwen_config.py:61) and its runner is wired to one model.
@@ -47,6 +48,8 @@ def unregister_architecture(name: str) -> None:
 
 def architecture_of(data: Mapping[str, Any]) -> Architecture:
     names = data.get("architectures")
+    if not names and isinstance(data.get("architecture"), str):
+        names = [data["architecture"]]  # configs that name their one architecture under the singular key
     if isinstance(names, (list, tuple)) and names:
         name = names[0]
         if name in ARCHITECTURES:

@@ -17,7 +17,8 @@ class PreNormBlock(Block):
 
     src/mini_llm_runtime/qwen_model_runner.py:198-218.  The residual stream is kept
     in 32-bit; each addition is fused into the norm that follows it, so the block
-    hands its last output to the next block (or the model) un-added.
+    hands its last output to the next block (or the model) un-added.  A layer without a
+    feed-forward (`feed_forward` None) is its first half only and needs only the "input" norm.
     """
 
     replayable = True
@@ -25,22 +26,22 @@ class PreNormBlock(Block):
 
     norm_names = ("input", "post_mixer")
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, norms: Mapping[str, Norm]) -> None:
-        missing = [n for n in self.norm_names if n not in norms]
+    def __init__(self, mixer: Mixer, feed_forward: Optional[FeedForward], norms: Mapping[str, Norm]) -> None:
+        needed = self.norm_names if feed_forward is not None else self.norm_names[:1]
+        missing = [n for n in needed if n not in norms]
         if missing:
-            raise ValueError(f"pre_norm block needs the norms {self.norm_names}, missing {missing}")
+            raise ValueError(f"pre_norm block needs the norms {needed}, missing {missing}")
         self.mixer = mixer
         self.feed_forward = feed_forward
         self.norm_input = norms["input"]
-        self.norm_post_mixer = norms["post_mixer"]
+        self.norm_post_mixer = norms["post_mixer"] if feed_forward is not None else None
 
     def children(self) -> dict[str, Part]:
-        return {
-            "mixer": self.mixer,
-            "feed_forward": self.feed_forward,
-            "norm_input": self.norm_input,
-            "norm_post_mixer": self.norm_post_mixer,
-        }
+        parts: dict[str, Part] = {"mixer": self.mixer, "norm_input": self.norm_input}
+        if self.feed_forward is not None:
+            parts["feed_forward"] = self.feed_forward
+            parts["norm_post_mixer"] = self.norm_post_mixer
+        return parts
 
     def forward(
         self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor], site: int
@@ -48,6 +49,8 @@ class PreNormBlock(Block):
         h = _norm(self.norm_input, self.mixer, ctx, x, delta)
         mixed = self.mixer.forward(ctx, h, site)
         x = _stream_after(h, x)
+        if self.feed_forward is None:
+            return x, mixed
         h = _norm(self.norm_post_mixer, self.feed_forward, ctx, x, mixed)
         out = self.feed_forward.forward(ctx, h)
         return _stream_after(h, x), out

@@ -43,3 +43,116 @@ class SwiGLU(FeedForward):
         ops = ctx.ops
         hidden = ops.linear(h, self.gate_up_weight, None, swiglu=True)
         return ops.linear(hidden, self.down_weight, None, for_stream=True)  # the next norm's delta
+
+
+ACTIVATIONS = ("relu2", "sigmoid")  # what `ops.linear(..., activation=)` applies to its sums
+
+
+@register_part("feed_forward", "mlp")
+class MLP(FeedForward):
+    """Dense feed-forward without a gate: `down(act(up(x)))`, no biases.  `activation` is applied
+    in the epilogue of the first product; "relu2" is max(z, 0)^2."""
+
+    replayable = True
+    takes_pending_norm = True  # `h` goes to the up product only
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "relu2") -> None:
+        if hidden_size <= 0 or intermediate_size <= 0:
+            raise ValueError("MLP sizes must be > 0")
+        if activation not in ACTIVATIONS:
+            raise ValueError(f"unknown activation {activation!r}; known: {', '.join(ACTIVATIONS)}")
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        self.activation = activation
+        self.up_weight: Optional[torch.Tensor] = None
+        self.down_weight: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {
+            "up_weight": ParamSpec((self.intermediate_size, self.hidden_size)),
+            "down_weight": ParamSpec((self.hidden_size, self.intermediate_size)),
+        }
+
+    def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
+        ops = ctx.ops
+        hidden = ops.linear(h, self.up_weight, None, activation=self.activation)
+        return ops.linear(hidden, self.down_weight, None, for_stream=True)  # the next norm's delta
+
+
+@register_part("feed_forward", "routed_experts")
+class RoutedExperts(FeedForward):
+    """A mixture of `experts` small feed-forwards (`down_e(act(up_e(x)))`, no biases) of which every
+    token uses `top`.
+
+    Routing, all in 32-bit: z = Wr h; s = sigmoid(z); the choice is made on c = s + correction (a
+    stored vector that steers the load and takes no part in the weights).  The experts form
+    `groups` equal groups of neighbours; a group's score is the sum of its two largest c, only
+    experts of the `keep_groups` best groups can be chosen (for the others c counts as minus
+    infinity), and of those the `top` largest c win.  A chosen expert's output is weighted with
+    its s times `router_scale`; the weights are not renormalised.
+
+    Everything runs on the device, so steps can be recorded: the routing kernel leaves expert ids
+    and weights per token, an alignment kernel sorts the (token, choice) pairs by expert into row
+    tiles, and two grouped products run over those tiles (up with the activation, down with the
+    pair's weight).  The result is a float32 stack [top, tokens, hidden] of the weighted expert
+    outputs, which the next norm adds to the stream in that fixed order.
+    Expert matrices are stacked along the rows: up [experts * inner, hidden], down [experts *
+    hidden, inner].
+    """
+
+    replayable = True
+
+    def __init__(
+        self,
+        hidden_size: int,
+        intermediate_size: int,
+        experts: int,
+        top: int,
+        router_scale: float = 1.0,
+        groups: int = 1,
+        keep_groups: int = 1,
+        activation: str = "relu2",
+    ) -> None:
+        if hidden_size <= 0 or intermediate_size <= 0 or experts <= 0 or top <= 0:
+            raise ValueError("RoutedExperts sizes must be > 0")
+        if groups <= 0 or experts % groups or not 0 < keep_groups <= groups:
+            raise ValueError("the experts must divide into equal groups, of which 1..groups are kept")
+        if top > keep_groups * (experts // groups):
+            raise ValueError("the kept groups hold fewer experts than a token uses")
+        if activation not in ACTIVATIONS:
+            raise ValueError(f"unknown activation {activation!r}; known: {', '.join(ACTIVATIONS)}")
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        self.experts = int(experts)
+        self.top = int(top)
+        self.router_scale = float(router_scale)
+        self.groups = int(groups)
+        self.keep_groups = int(keep_groups)
+        self.activation = activation
+        self.router_weight: Optional[torch.Tensor] = None
+        self.correction: Optional[torch.Tensor] = None
+        self.up_weight: Optional[torch.Tensor] = None
+        self.down_weight: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {
+            "router_weight": ParamSpec((self.experts, self.hidden_size)),
+            "correction": ParamSpec((self.experts,), keep_stored_precision=True),
+            "up_weight": ParamSpec((self.experts * self.intermediate_size, self.hidden_size)),
+            "down_weight": ParamSpec((self.experts * self.hidden_size, self.intermediate_size)),
+        }
+
+    def bind(self, params, *, dtype: torch.dtype, device: torch.device) -> None:
+        super().bind(params, dtype=dtype, device=device)
+        self.correction = self.correction.to(torch.float32)  # the routing is 32-bit throughout
+
+    def forward(self, ctx: StepContext, h: torch.Tensor):
+        ops = ctx.ops
+        logits = ops.linear(h, self.router_weight, None, out_dtype=torch.float32)
+        ids, weights = ops.route_experts(
+            logits, self.correction, top=self.top, groups=self.groups, keep_groups=self.keep_groups,
+            scale=self.router_scale,
+        )
+        return ops.expert_products(
+            h, self.up_weight, self.down_weight, ids, weights, experts=self.experts, activation=self.activation
+        )

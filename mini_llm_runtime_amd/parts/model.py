@@ -19,7 +19,7 @@ from .spec import LayerSpec, ModelSpec, ParamSpec, PartSpec
 
 def _build_layer(spec: LayerSpec) -> Block:
     mixer = build_part("mixer", spec.mixer)
-    feed_forward = build_part("feed_forward", spec.feed_forward)
+    feed_forward = build_part("feed_forward", spec.feed_forward) if spec.feed_forward is not None else None
     norms = {name: build_part("norm", s) for name, s in spec.norms.items()}
     return build_part("block", PartSpec(spec.block), mixer=mixer, feed_forward=feed_forward, norms=norms)
 

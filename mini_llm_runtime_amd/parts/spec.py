@@ -36,11 +36,12 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: an arrangement (`block`) of a mixer, a feed-forward and norms."""
+    """One layer: an arrangement (`block`) of a mixer, a feed-forward (None: the layer has
+    none, if its arrangement allows that) and norms."""
 
     block: str
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: Optional[PartSpec]
     norms: Mapping[str, PartSpec]
 
 

@@ -51,11 +51,22 @@ class TorchOps:
         return (x[:, rows.long()] if x.dim() == 3 else x[rows.long()]).contiguous()
 
     # matrix products ---------------------------------------------------------------------
-    def linear(self, x, weight, bias=None, out_dtype=None, kernel="auto", swiglu=False, partial_sums=False, for_stream=False):
+    def linear(
+        self, x, weight, bias=None, out_dtype=None, kernel="auto", swiglu=False, partial_sums=False, for_stream=False,
+        activation=None, multiply=None,
+    ):
         self._count("linear")
         y = x.float() @ weight.float().t()
         if bias is not None:
             y = y + bias.float()
+        if activation == "relu2":
+            y = torch.clamp(y, min=0.0) ** 2
+        elif activation == "sigmoid":
+            y = torch.sigmoid(y)
+        elif activation is not None:
+            raise ValueError(activation)
+        if multiply is not None:
+            y = y * multiply.float()
         if swiglu:  # rows of weight: gate 2j, gate 2j+1, up 2j, up 2j+1
             quads = y.view(y.shape[0], -1, 4)
             gate, up = quads[..., :2], quads[..., 2:]
@@ -108,7 +119,7 @@ class TorchOps:
 
     def paged_attention(
         self, qkv, key_pages, value_pages, block_table, ctx, *, num_heads, num_kv_heads, head_dim, block_size, scale, window,
-        defer_merge=False, plan=None,
+        defer_merge=False, plan=None, chunk=None,
     ):
         self._count("paged_attention")
         tokens = qkv.shape[0]
@@ -120,6 +131,8 @@ class TorchOps:
             r = int(ctx.token_entry[t])
             p = int(ctx.positions[t])
             first = 0 if window is None else max(0, p - window + 1)
+            if chunk is not None:
+                first = p // chunk * chunk
             idx = torch.arange(first, p + 1)
             page = table[r, idx // block_size]
             assert (page >= 0).all(), "attention would read a page that is not there"
@@ -131,6 +144,40 @@ class TorchOps:
             w = torch.softmax(s, dim=-1)
             out[t] = torch.einsum("hn,nhd->hd", w, v)
         return out.reshape(tokens, num_heads * head_dim).to(self.dtype)
+
+    # routed experts ------------------------------------------------------------------------------
+    def route_experts(self, logits, correction, *, top, groups, keep_groups, scale):
+        self._count("route_experts")
+        tokens, experts = logits.shape
+        s = torch.sigmoid(logits.float())
+        c = s + correction.float()
+        per = experts // groups
+        ids = torch.empty(tokens, top, dtype=torch.int32)
+        weights = torch.empty(tokens, top, dtype=torch.float32)
+        for t in range(tokens):
+            score = [sum(sorted(c[t, g * per : (g + 1) * per].tolist(), reverse=True)[:2]) for g in range(groups)]
+            kept = sorted(range(groups), key=lambda g: (-score[g], g))[:keep_groups]
+            allowed = [e for e in range(experts) if e // per in kept]
+            chosen = sorted(allowed, key=lambda e: (-float(c[t, e]), e))[:top]
+            for j, e in enumerate(chosen):
+                ids[t, j] = e
+                weights[t, j] = s[t, e] * scale
+        return ids.to(logits.device), weights.to(logits.device)
+
+    def expert_products(self, h, up_weight, down_weight, ids, weights, *, experts, activation):
+        self._count("expert_products")
+        tokens, hidden = h.shape
+        top = ids.shape[1]
+        up = up_weight.float().view(experts, -1, hidden)
+        down = down_weight.float().view(experts, hidden, -1)
+        out = torch.zeros(top, tokens, hidden, dtype=torch.float32, device=h.device)
+        for t in range(tokens):
+            for j in range(top):
+                e = int(ids[t, j])
+                z = up[e] @ h[t].float()
+                a = torch.clamp(z, min=0.0) ** 2 if activation == "relu2" else torch.sigmoid(z)
+                out[j, t] = weights[t, j] * (down[e] @ a.to(self.dtype).float())
+        return out
 
     # sampling ----------------------------------------------------------------------------------
     def sample(self, logits, temperature: Optional[torch.Tensor], uniform: Optional[torch.Tensor]):
