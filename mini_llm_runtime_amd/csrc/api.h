@@ -71,8 +71,12 @@ int mlr_qkv_finish(const float* partial, int slices, const float* cos, const flo
 // Plain 32-bit FMA arithmetic on every path (no matrix-core rounding).
 // With `swiglu` the rows of w come in groups (gate 2j, gate 2j+1, up 2j, up 2j+1),
 // there is no bias, n is a multiple of 4 and y[M, N / 2] = silu(gate) * up.
+// `swiglu` 2 and 3 are element-wise activations instead: the squared ReLU max(v, 0)^2 and the
+// sigmoid, applied after the bias, any n.  `multiply` ([M, N] in `dtype`, or null; not with the
+// pairing) is multiplied into the activated sums: y = act(x w^T + bias) * multiply.
 int mlr_gemm_simple(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
-                    int out_is_f32, int swiglu, int dtype, int m, int n, int k, hipStream_t stream);
+                    int out_is_f32, int swiglu, int dtype, int m, int n, int k, const void* multiply,
+                    hipStream_t stream);
 
 // The same product in bfloat16 on the matrix cores (float32 accumulation).  Needs
 // k % 8 == 0 and 16-byte aligned x and w; any m and n.  With slices > 1 (a value
@@ -93,7 +97,8 @@ int mlr_gemm_bf16_kernel(int m, int n, int k, int slices);
 // sums of row i are scaled by rsqrt(sum_p row_sumsq[i, p] / k + norm_eps) before the bias.
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
                   int out_is_f32, int swiglu, int slices, int kernel, int m, int n, int k,
-                  const float* row_sumsq, int sumsq_parts, float norm_eps, hipStream_t stream);
+                  const float* row_sumsq, int sumsq_parts, float norm_eps, const void* multiply,
+                  hipStream_t stream);
 
 // A product that finishes the residual stream (gemm_stream.hip): y = a w^T (+ bias), a [m, k] and w
 // [n, k] bfloat16; then, every workgroup for its own columns of all rows, stream[m, n] (float32, in
@@ -145,7 +150,8 @@ int mlr_gemm_merge_fused_bf16(const float* attn_partial, const int* context_lens
 
 // Attention of every token over its request's pages: token t (entry
 // token_entry[t], absolute position positions[t]) sees the keys
-// max(0, p - window + 1) .. p of its entry's block table row (window 0: all).
+// max(0, p - window + 1) .. p of its entry's block table row (window 0: all), or, with a
+// chunked mask (chunk > 0, window 0), the keys p - p % chunk .. p.
 // q is read from q[t * q_stride + head * head_dim + i]; out is [tokens, heads * head_dim];
 // pages are laid out as for mlr_rope_kv_write.
 // A page id outside [0, num_pages) among the visible keys gives a NaN row.
@@ -153,7 +159,7 @@ int mlr_paged_attention_simple(const void* q, int64_t q_stride, const void* key_
                                const void* value_pages, const int* block_table, int table_width,
                                const int* token_entry, const int* positions, void* out, int dtype,
                                int tokens, int entries, int heads, int kv_heads, int head_dim,
-                               int block_size, int num_pages, float scale, int window,
+                               int block_size, int num_pages, float scale, int window, int chunk,
                                hipStream_t stream);
 
 // tokens[k] = argmax(logits[k, :]) (first maximum), or, where temperature[k] > 0,
@@ -176,5 +182,28 @@ int mlr_sample(const float* logits, const float* temperature, const float* unifo
 int64_t mlr_sample_static_capacity();
 int mlr_sample_static(const float* logits, const float* temperature, const float* uniform, int* tokens,
                       int rows, int vocab, hipStream_t stream);
+
+// Routed experts (moe.hip).  mlr_moe_route: per token, from the router's float32 logits [tokens,
+// experts]: s = sigmoid(z), choice scores c = s + correction (float32 [experts], or null); the
+// experts form `groups` equal groups of neighbours, a group's score is the sum of its two largest
+// c, only experts of the `keep` best groups can be chosen; ids [tokens, top] are the `top` largest
+// c among those (ties to the lower index) and weights [tokens, top] their s times `scale`.
+int mlr_moe_route(const float* logits, const float* correction, int* ids, float* weights, int tokens, int experts,
+                  int top, int groups, int keep, float scale, hipStream_t stream);
+// The (token, choice) pairs p = token * top + choice sorted by expert: sorted [pairs], offsets
+// [experts + 1], tiles [max_tiles, 2] = (expert, first row of `sorted`) with up to
+// mlr_moe_tile_rows() rows each, unused tiles (-1, 0).  max_tiles >= mlr_moe_max_tiles(pairs, experts).
+int mlr_moe_tile_rows();
+int mlr_moe_max_tiles(int pairs, int experts);
+int mlr_moe_align(const int* ids, int pairs, int experts, int max_tiles, int* sorted, int* offsets, int* tiles,
+                  hipStream_t stream);
+// One grouped product over those tiles; w is [experts, n, k] in `dtype` (0 float32, 1 bfloat16).
+// up 1: a = h [tokens, k]; out [pairs, n] in `dtype`, row r = act(h[sorted[r] / top] w[e]^T), act 0
+// none, 2 squared ReLU, 3 sigmoid.  up 0: a = the rows of the first product [pairs, k]; out float32
+// [top, tokens, n], out[choice, token] = pair_weights[p] * (a[r] w[e]^T).  mfma 1: on the matrix
+// cores (bfloat16, k % 8 == 0), else plain 32-bit FMA arithmetic.
+int mlr_moe_gemm(const void* a, const void* w, const int* sorted, const int* offsets, const int* tiles,
+                 const float* pair_weights, void* out, int up, int dtype, int mfma, int max_tiles, int tokens, int top,
+                 int n, int k, int act, hipStream_t stream);
 
 }  // extern "C"

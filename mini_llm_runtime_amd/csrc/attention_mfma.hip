@@ -164,7 +164,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out,
     float* __restrict__ partial, int heads, int kv_heads, int head_tiles, int block_size, int num_pages,
-    float scale, int window, int part, int splits) {
+    float scale, int window, int chunk, int part, int splits) {
   __shared__ float sm_acc[kDecodeWaves][16][D];
   __shared__ float sm_m[kDecodeWaves][16];
   __shared__ float sm_l[kDecodeWaves][16];
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
 
   const int ctx = context_lens[entry];
   const int p = ctx - 1;
-  const int first = window > 0 ? max(0, p - window + 1) : 0;
+  const int first = first_visible_key(p, window, chunk);
   const int base = (first / 16) * 16;
   const int kb = base + split * part;
   const int ke = min(kb + part, ctx);
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
                                                                   const int* __restrict__ cu_q,
                                                                   const int* __restrict__ context_lens,
                                                                   bf16* __restrict__ out, int heads, int window,
-                                                                  int part, int all_splits) {
+                                                                  int chunk, int part, int all_splits) {
   const int entry = blockIdx.x;
   const int h = blockIdx.y;
   const int lane = threadIdx.x;
@@ -345,7 +345,7 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
   const float* src = partial + (static_cast<int64_t>(entry) * heads + h) * all_splits * kPartialStride;
   // the partitions that hold keys of this entry (the others wrote nothing), as attn_decode cuts them
   const int ctx = context_lens[entry];
-  const int first = window > 0 ? max(0, ctx - window) : 0;
+  const int first = first_visible_key(ctx - 1, window, chunk);
   const int splits = min(all_splits, (ctx - (first / 16) * 16 + part - 1) / part);
   // The numerators are read kMergeBatch partitions at a time, all loads of a batch issued
   // before the first is used, and the first batch before the reductions below: this kernel's
@@ -456,7 +456,7 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, const int* __restrict__ cu_q, const int* __restrict__ context_lens,
     bf16* __restrict__ out, int num_tiles, int heads, int kv_heads, int bs_shift, int num_pages, float scale,
-    int window, float* __restrict__ partial) {
+    int window, int chunk, float* __restrict__ partial) {
   // gridDim.y > 1: the keys of every tile are cut into that many runs, one workgroup each, which
   // leave their unnormalised results in `partial` for attn_prefill_merge (few tiles behind a long
   // context would otherwise be as many long chains on a few compute units).
@@ -515,7 +515,7 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     qi[b] = q0 + wave * kWaveQ + b * 16 + col;
     q_ok[b] = qi[b] < q_len;
     pq[b] = pos0 + qi[b];  // its absolute position
-    pq_first[b] = window > 0 ? max(0, pq[b] - window + 1) : 0;
+    pq_first[b] = first_visible_key(pq[b], window, chunk);
     qo[b] = load_row(q + static_cast<int64_t>(t_first + (q_ok[b] ? qi[b] : 0)) * q_stride + static_cast<int64_t>(head) * D,
                      q_ok[b], quarter);
   }
@@ -523,7 +523,7 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   // key range of the workgroup: from the first query's window start to the last query's position
   const int last_q = min(q0 + kWgQ, q_len) - 1;
   const int k_end = pos0 + last_q + 1;
-  const int k_begin_raw = window > 0 ? max(0, pos0 + q0 - window + 1) : 0;
+  const int k_begin_raw = first_visible_key(pos0 + q0, window, chunk);
   const int k_begin_all = (k_begin_raw / kTileK) * kTileK;
   // this workgroup's run of the keys: whole turns of the loop below (all key groups together)
   constexpr int kTurn = kKeyGroups * kTileK;
@@ -534,12 +534,12 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   const int k_stop = min(k_end, k_begin + turns_each * kTurn);  // keys from here on belong to the next run
   // the wavefront's own range (uniform within the wavefront)
   const int w_last = pos0 + min(q0 + wave * kWaveQ + kWaveQ - 1, q_len - 1);
-  const int w_first = window > 0 ? max(0, pos0 + q0 + wave * kWaveQ - window + 1) : 0;
+  const int w_first = first_visible_key(pos0 + q0 + wave * kWaveQ, window, chunk);
   const bool wave_has_queries = q0 + wave * kWaveQ < q_len;
   // a tile is fully visible to the wavefront when it ends at or before its first query's position
   // and starts at or after its last query's window start (queries beyond q_len are never stored)
   const int w_min_pos = pos0 + q0 + wave * kWaveQ;
-  const int w_max_first = window > 0 ? max(0, pos0 + q0 + wave * kWaveQ + kWaveQ - 1 - window + 1) : 0;
+  const int w_max_first = first_visible_key(pos0 + q0 + wave * kWaveQ + kWaveQ - 1, window, chunk);
   // softmax in base 2: exp(x) = exp2(x * log2(e))
   const float scale2 = scale * 1.44269504088896340736f;
 
@@ -613,7 +613,7 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
       if (!in) bad = bad || (k_row[i] < lim && kt0 + k_row[i] >= k_begin_raw);
       t.k[i] = load_bf16x8(key_pages + (static_cast<uint64_t>(in ? static_cast<uint32_t>(page) : 0u) * page_elems + k_in_page[i]));
     }
-    const bool guard = lim < kTileK || window > 0;  // uniform
+    const bool guard = lim < kTileK || window > 0 || chunk > 0;  // uniform
 #pragma unroll
     for (int i = 0; i < kPieces; ++i) {
       const int page = v_ids[i];
@@ -903,7 +903,7 @@ int64_t mlr_attention_decode_scratch(int entries, int heads, int splits) {
 int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages, const void* value_pages,
                          const int* block_table, int table_width, const int* cu_q, const int* context_lens,
                          void* out, float* partial, int entries, int heads, int kv_heads, int block_size,
-                         int num_pages, float scale, int window, int part, int splits, int merge,
+                         int num_pages, float scale, int window, int chunk, int part, int splits, int merge,
                          hipStream_t stream) {
   MLR_REQUIRE(q && key_pages && value_pages && block_table && cu_q && context_lens && out, "null pointer");
   MLR_REQUIRE(entries > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "bad head counts");
@@ -916,7 +916,8 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
   MLR_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(key_pages) % 16 == 0 &&
                   reinterpret_cast<uintptr_t>(value_pages) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
               "operands must be 16-byte aligned");
-  MLR_REQUIRE(scale > 0.f && scale < INFINITY && window >= 0, "bad scale or window");
+  MLR_REQUIRE(scale > 0.f && scale < INFINITY && window >= 0 && chunk >= 0 && !(window > 0 && chunk > 0),
+              "bad scale, window or chunk");
   const int group = heads / kv_heads;
   const int head_tiles = (group + 15) / 16;
   MLR_REQUIRE(kv_heads * head_tiles <= 65535, "too many heads for one launch");
@@ -929,7 +930,7 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
 #define MLR_DECODE(depth)                                                                                       \
   attn_decode_kernel<depth><<<grid, kDecodeWaves * kWave, 0, stream>>>(                                         \
       qp, q_stride, kp, vp, block_table, table_width, cu_q, context_lens, op, partial, heads, kv_heads,         \
-      head_tiles, block_size, num_pages, scale, window, part, splits)
+      head_tiles, block_size, num_pages, scale, window, chunk, part, splits)
   bool launched = false;
   if constexpr (kMaxDecodeDepth >= 4) {
     if (tiles_per_wave >= 4) {
@@ -948,7 +949,7 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
   MLR_LAUNCH_CHECK();
   if (splits > 1 && merge) {
     attn_decode_merge_kernel<<<dim3(entries, heads), kWave, 0, stream>>>(
-        partial, cu_q, context_lens, static_cast<bf16*>(out), heads, window, part, splits);
+        partial, cu_q, context_lens, static_cast<bf16*>(out), heads, window, chunk, part, splits);
     MLR_LAUNCH_CHECK();
   }
   return 0;
@@ -957,12 +958,12 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
 // The merge that mlr_attention_decode left out: out[t] of every single-token entry from its
 // partitions in `partial`.
 int mlr_attention_decode_merge(const float* partial, const int* cu_q, const int* context_lens, void* out, int entries,
-                               int heads, int window, int part, int splits, hipStream_t stream) {
+                               int heads, int window, int chunk, int part, int splits, hipStream_t stream) {
   MLR_REQUIRE(partial && cu_q && context_lens && out, "null pointer");
   MLR_REQUIRE(entries > 0 && heads > 0 && heads <= 65535, "bad sizes");
-  MLR_REQUIRE(part > 0 && part % 64 == 0 && splits > 1 && window >= 0, "bad partitions");
+  MLR_REQUIRE(part > 0 && part % 64 == 0 && splits > 1 && window >= 0 && chunk >= 0, "bad partitions");
   attn_decode_merge_kernel<<<dim3(entries, heads), kWave, 0, stream>>>(partial, cu_q, context_lens,
-                                                                      static_cast<bf16*>(out), heads, window, part, splits);
+                                                                      static_cast<bf16*>(out), heads, window, chunk, part, splits);
   MLR_LAUNCH_CHECK();
   return 0;
 }
@@ -986,8 +987,8 @@ int64_t mlr_attention_prefill_scratch(int num_tiles, int heads, int splits, int 
 int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages, const void* value_pages,
                           const int* block_table, int table_width, const int* tiles, int num_tiles, int wide,
                           const int* cu_q, const int* context_lens, void* out, int heads, int kv_heads,
-                          int block_size, int num_pages, float scale, int window, int splits, float* partial,
-                          hipStream_t stream) {
+                          int block_size, int num_pages, float scale, int window, int chunk, int splits,
+                          float* partial, hipStream_t stream) {
   MLR_REQUIRE(splits >= 1 && splits <= 64, "splits must lie within 1..64");
   MLR_REQUIRE(splits == 1 || partial != nullptr, "several key runs need scratch memory");
   MLR_REQUIRE(q && key_pages && value_pages && block_table && tiles && cu_q && context_lens && out, "null pointer");
@@ -1003,7 +1004,8 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
   MLR_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(key_pages) % 16 == 0 &&
                   reinterpret_cast<uintptr_t>(value_pages) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
               "operands must be 16-byte aligned");
-  MLR_REQUIRE(scale > 0.f && scale < INFINITY && window >= 0, "bad scale or window");
+  MLR_REQUIRE(scale > 0.f && scale < INFINITY && window >= 0 && chunk >= 0 && !(window > 0 && chunk > 0),
+              "bad scale, window or chunk");
   MLR_REQUIRE(static_cast<int64_t>(num_tiles) * heads < (1ll << 31), "too many tiles for one launch");
   static bool configured = false;
   if (!configured) {
@@ -1030,12 +1032,12 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
       attn_prefill_kernel<qb, true><<<grid, 256 * kKeyGroups, kPrefillLds, stream>>>(                         \
           static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),                         \
           static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,         \
-          static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window, partial);  \
+          static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window, chunk, partial);  \
     else                                                                                                      \
       attn_prefill_kernel<qb, false><<<grid, 256 * kKeyGroups, kPrefillLds, stream>>>(                        \
           static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),                         \
           static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,         \
-          static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window, partial);  \
+          static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window, chunk, partial);  \
   } while (0)
   if constexpr (D <= 128) {
     if (wide)

@@ -21,7 +21,7 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ key_pages,
     const T* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ token_entry, const int* __restrict__ positions, T* __restrict__ out, int entries,
-    int heads, int kv_heads, int head_dim, int block_size, int num_pages, float scale, int window) {
+    int heads, int kv_heads, int head_dim, int block_size, int num_pages, float scale, int window, int chunk) {
   __shared__ float qs[kMaxHeadDim];
   __shared__ float ps[kWave];
   __shared__ int64_t offs[kWave];
@@ -44,7 +44,7 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
   __syncthreads();
 
   const int* table = block_table + static_cast<int64_t>(entry) * table_width;
-  const int first = window > 0 ? max(0, p - window + 1) : 0;
+  const int first = first_visible_key(p, window, chunk);
   float m = -INFINITY;
   float l = 0.f;
   float acc[kMaxHeadDim / kWave] = {0.f, 0.f, 0.f, 0.f};
@@ -113,7 +113,7 @@ extern "C" int mlr_paged_attention_simple(const void* q, int64_t q_stride, const
                                           const void* value_pages, const int* block_table, int table_width,
                                           const int* token_entry, const int* positions, void* out, int dtype,
                                           int tokens, int entries, int heads, int kv_heads, int head_dim,
-                                          int block_size, int num_pages, float scale, int window,
+                                          int block_size, int num_pages, float scale, int window, int chunk,
                                           hipStream_t stream) {
   MLR_REQUIRE(q && key_pages && value_pages && block_table && token_entry && positions && out, "null pointer");
   MLR_REQUIRE(tokens > 0 && entries > 0 && heads > 0 && kv_heads > 0, "sizes must be > 0");
@@ -122,7 +122,7 @@ extern "C" int mlr_paged_attention_simple(const void* q, int64_t q_stride, const
   MLR_REQUIRE(block_size > 0 && num_pages > 0 && table_width > 0, "page sizes must be > 0");
   MLR_REQUIRE(q_stride >= static_cast<int64_t>(heads) * head_dim, "q_stride is smaller than a row of queries");
   MLR_REQUIRE(scale > 0.f && scale < INFINITY, "scale must be positive and finite");
-  MLR_REQUIRE(window >= 0, "window must be >= 0");
+  MLR_REQUIRE(window >= 0 && chunk >= 0 && !(window > 0 && chunk > 0), "a window or a chunked mask, each >= 0");
   MLR_REQUIRE(heads < 65536, "too many heads for one launch");
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
   dim3 grid(tokens, heads);
@@ -130,12 +130,12 @@ extern "C" int mlr_paged_attention_simple(const void* q, int64_t q_stride, const
     paged_attention_simple_kernel<float><<<grid, kWave, 0, stream>>>(
         static_cast<const float*>(q), q_stride, static_cast<const float*>(key_pages),
         static_cast<const float*>(value_pages), block_table, table_width, token_entry, positions,
-        static_cast<float*>(out), entries, heads, kv_heads, head_dim, block_size, num_pages, scale, window);
+        static_cast<float*>(out), entries, heads, kv_heads, head_dim, block_size, num_pages, scale, window, chunk);
   else
     paged_attention_simple_kernel<bf16><<<grid, kWave, 0, stream>>>(
         static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),
         static_cast<const bf16*>(value_pages), block_table, table_width, token_entry, positions,
-        static_cast<bf16*>(out), entries, heads, kv_heads, head_dim, block_size, num_pages, scale, window);
+        static_cast<bf16*>(out), entries, heads, kv_heads, head_dim, block_size, num_pages, scale, window, chunk);
   MLR_LAUNCH_CHECK();
   return 0;
 }

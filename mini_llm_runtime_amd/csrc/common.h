@@ -81,6 +81,14 @@ __device__ __forceinline__ float lane_value(float v, int lane) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
 
+// The first key a query at position p sees (the last one is p itself): all of them; with a
+// window only the `window` most recent; with a chunked mask only those of its own run of
+// `chunk` positions, runs counted from position 0 of the request.
+__host__ __device__ inline int first_visible_key(int p, int window, int chunk) {
+  if (chunk > 0) return p - p % chunk;
+  return window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
+}
+
 __device__ inline float wave_sum(float v) {
   v += dpp_move<0x121>(v);  // row_ror:1
   v += dpp_move<0x122>(v);  // row_ror:2

@@ -13,7 +13,10 @@ struct GemmEpilogue {
   int bias_is_f32;
   void* y;
   int out_is_f32;
-  int swiglu;  // store silu(v0) * v2, silu(v1) * v3 into a row of N / 2
+  // What happens to the sums before they are stored (the entry points call this `swiglu`, its
+  // first meaning): kEpSwiglu stores silu(v0) * v2, silu(v1) * v3 into a row of N / 2; kEpRelu2
+  // stores max(v, 0)^2 and kEpSigmoid 1 / (1 + exp(-v)), element by element, after the bias.
+  int swiglu;
   // Rows whose normalisation is still owed (see gemm_stream.hip): x holds weight * stream, not yet
   // divided by the root mean square of the stream.  The sums of a row m are then scaled by
   // rsqrt(sum_p row_sumsq[m, p] / K + eps) before the bias: the factor is the same for the whole
@@ -21,7 +24,15 @@ struct GemmEpilogue {
   const float* row_sumsq = nullptr;  // [M, sumsq_parts]: partial sums of squares of every stream row
   int sumsq_parts = 0;
   float norm_eps = 0.f;
+  // [M, N] bfloat16, or null: the stored value is the (activated) sum times this, element by element
+  // (a gate: sigmoid(x Wg^T) * other).  Not with kEpSwiglu, not with partial sums.
+  const void* multiply = nullptr;
 };
+
+constexpr int kEpNone = 0;
+constexpr int kEpSwiglu = 1;
+constexpr int kEpRelu2 = 2;
+constexpr int kEpSigmoid = 3;
 
 // The scaling factors of rows m0 .. m0 + count - 1 into `scales` (LDS), by all wavefronts of the
 // workgroup (a whole number of them): wavefront w takes the rows w, w + waves, ..., its lanes the
@@ -101,7 +112,7 @@ __device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g));
 __device__ __forceinline__ void store4(const GemmEpilogue& ep, int64_t m, int n, int N, float v0, float v1,
                                        float v2, float v3) {
   float v[4] = {v0, v1, v2, v3};
-  if (ep.swiglu) {
+  if (ep.swiglu == kEpSwiglu) {
     // n..n+3 = gate 2j, gate 2j+1, up 2j, up 2j+1 with j = n / 4; N is a multiple of 4
     const int64_t at = m * (N / 2) + n / 2;
     const float a = silu(v[0]) * v[2];
@@ -123,6 +134,22 @@ __device__ __forceinline__ void store4(const GemmEpilogue& ep, int64_t m, int n,
       if (n + i < N) v[i] += load_as_f32(ep.bias, n + i, ep.bias_is_f32);
   }
   const int64_t at = m * N + n;
+  if (ep.swiglu == kEpRelu2) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float r = fmaxf(v[i], 0.f);
+      v[i] = r * r;
+    }
+  } else if (ep.swiglu == kEpSigmoid) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = 1.0f / (1.0f + __expf(-v[i]));
+  }
+  if (ep.multiply != nullptr) {
+    const bf16* other = static_cast<const bf16*>(ep.multiply) + at;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n + i < N) v[i] *= to_f32(other[i]);
+  }
   if (ep.out_is_f32) {
     float* y = static_cast<float*>(ep.y) + at;
     if (n + 3 < N && (at & 3) == 0) {

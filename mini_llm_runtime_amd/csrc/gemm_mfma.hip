@@ -1130,21 +1130,26 @@ int mlr_gemm_bf16_kernel(int m, int n, int k, int slices) { return choose_kernel
 // a multiple of 4 and y is [m, n / 2].  With slices > 1 (the value of
 // mlr_gemm_bf16_slices; not with swiglu) y is float32 [slices, m, n]: partial sums
 // over slices of k, the bias in slice 0, for the consumer to add up.
+// `swiglu` 2 and 3 are element-wise activations instead (squared ReLU, sigmoid; any n, after the
+// bias), and `multiply` (bfloat16 [m, n], or null) is multiplied into the activated sums.
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y, int out_is_f32,
                   int swiglu, int slices, int kernel, int m, int n, int k, const float* row_sumsq, int sumsq_parts,
-                  float norm_eps, hipStream_t stream) {
+                  float norm_eps, const void* multiply, hipStream_t stream) {
   MLR_REQUIRE(x && w && y, "null pointer");
+  MLR_REQUIRE(swiglu >= kEpNone && swiglu <= kEpSigmoid, "unknown epilogue");
+  MLR_REQUIRE(multiply == nullptr || (swiglu != kEpSwiglu && slices == 1), "a multiplier goes with whole, unpaired sums");
+  MLR_REQUIRE(slices == 1 || swiglu == kEpNone, "partial sums take no activation");
   MLR_REQUIRE(m > 0 && n > 0 && k > 0, "sizes must be > 0");
   MLR_REQUIRE(k % 8 == 0, "k must be a multiple of 8");
   MLR_REQUIRE(k <= (1 << 20), "k must not exceed 2^20 (32-bit byte offsets inside a tile)");
-  MLR_REQUIRE(!swiglu || (n % 4 == 0 && bias == nullptr), "swiglu needs n % 4 == 0 and no bias");
+  MLR_REQUIRE(swiglu != kEpSwiglu || (n % 4 == 0 && bias == nullptr), "swiglu needs n % 4 == 0 and no bias");
   MLR_REQUIRE(slices >= 1 && slices <= 64, "slices must be within 1..64");
   MLR_REQUIRE(slices == 1 || (!swiglu && out_is_f32), "partial sums are float32, without SwiGLU");
   MLR_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
               "x and w must be 16-byte aligned");
   MLR_REQUIRE(row_sumsq == nullptr || (sumsq_parts > 0 && sumsq_parts <= (1 << 16) && norm_eps >= 0.f),
               "sums of squares come with their number per row (1..65536) and an eps >= 0");
-  GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu, row_sumsq, sumsq_parts, norm_eps};
+  GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu, row_sumsq, sumsq_parts, norm_eps, multiply};
   if (kernel == 0) kernel = choose_kernel(m, n, k, slices);
   if (gemm_bf16(static_cast<const bf16*>(x), static_cast<const bf16*>(w), ep, m, n, k, slices, kernel, stream) != 0)
     return -1;

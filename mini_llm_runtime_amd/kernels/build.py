@@ -64,6 +64,7 @@ CORE = Module(
         "gemm_fused.hip",
         "gemm_stream.hip",
         "attention_simple.hip",
+        "moe.hip",
         "sampling.hip",
     ),
 )

@@ -37,8 +37,13 @@ _SIGNATURES = {
     "mlr_rope_table": ([_VP, _VP, _VP, _VP, _I, _I, _VP], _I),
     "mlr_rope_kv_write": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_qkv_finish": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
-    "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP], _I),
-    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _I, _VP, _I, _F, _VP], _I),
+    "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP], _I),
+    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _I, _VP, _I, _F, _VP, _VP], _I),
+    "mlr_moe_route": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _VP], _I),
+    "mlr_moe_tile_rows": ([], _I),
+    "mlr_moe_max_tiles": ([_I, _I], _I),
+    "mlr_moe_align": ([_VP, _I, _I, _I, _VP, _VP, _VP, _VP], _I),
+    "mlr_moe_gemm": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_residual_parts": ([_I, _I], _I),
     "mlr_gemm_residual_bf16": ([_VP, _VP, _VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _VP], _I),
     "mlr_gemm_bf16_slices": ([_I, _I, _I, _I], _I),
@@ -57,7 +62,7 @@ _SIGNATURES = {
     ),
     "mlr_gemm_merge_fused_bf16": ([_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I, _VP, _I, _I, _I, _I, _VP], _I),
     "mlr_paged_attention_simple": (
-        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP],
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _VP],
         _I,
     ),
     "mlr_sample": ([_VP, _VP, _VP, _VP, _VP, _I, _I, _VP], _I),
@@ -67,16 +72,19 @@ _SIGNATURES = {
     "mlr_attention_wide_tile": ([], _I),
     "mlr_attention_decode_scratch": ([_I, _I, _I], _I64),
     "mlr_attention_decode": (
-        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _VP],
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _VP],
         _I,
     ),
-    "mlr_attention_decode_merge": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_attention_decode_merge": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_attention_prefill_scratch": ([_I, _I, _I, _I], _I64),
     "mlr_attention_prefill": (
-        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _I, _VP, _VP],
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _I, _I, _VP, _VP],
         _I,
     ),
 }
+
+# what `linear` may do to its sums before it stores them (the entry points' `swiglu` argument)
+_EPILOGUES = {None: 0, "swiglu": 1, "relu2": 2, "sigmoid": 3}
 
 from .plans import PAGED_ATTENTION, QUERY_TILE, WIDE_QUERY_TILE, attention_plan, query_tiles  # noqa: F401
 
@@ -319,7 +327,7 @@ class HipOps:
             out = self._empty((h.tokens, h.heads * h.head_dim), self.dtype)
             self._call(
                 "mlr_attention_decode_merge", self._ptr(h.partial), self._ptr(h.cu_q), self._ptr(h.context_lens),
-                self._ptr(out), h.tokens, h.heads, h.window, h.part, h.splits, self._stream(), lib=h.library,
+                self._ptr(out), h.tokens, h.heads, h.window, 0, h.part, h.splits, self._stream(), lib=h.library,
             )
             return out
         return h
@@ -398,8 +406,15 @@ class HipOps:
         mfma_kernel: int = 0,
         slices: Optional[int] = None,
         for_stream: bool = False,
+        activation: Optional[str] = None,
+        multiply: Optional[torch.Tensor] = None,
     ) -> torch.Tensor:
         """x [M, K] times weight [N, K] transposed, plus bias [N]; F.linear semantics.
+
+        activation: "relu2" (max(v, 0)^2) or "sigmoid", applied to the sums (after the bias) in the
+        product's epilogue, in 32-bit, before the one rounding to the output's dtype.
+        multiply: [M, N] in the engine's dtype; the (activated) sums are multiplied with it element
+        by element before they are stored: a gate, sigmoid(x Wg^T) * other, in one kernel.
 
         for_stream: the result is a part's output and goes nowhere but into the next norm as its
         delta (as with partial_sums); it may then come back unrun, as a `PendingLinear` that the norm
@@ -418,6 +433,11 @@ class HipOps:
         """
         if kernel not in ("auto", "fma"):
             raise KernelError("kernel must be 'auto' or 'fma'")
+        if activation not in _EPILOGUES or activation == "swiglu":
+            raise KernelError(f"unknown activation {activation!r}")
+        if (activation is not None or multiply is not None) and (swiglu or partial_sums or for_stream or slices not in (None, 1)):
+            raise KernelError("an activation or a multiplier goes with whole sums: no SwiGLU pairing, no slices of k")
+        epilogue = 1 if swiglu else _EPILOGUES[activation]
         if for_stream:
             partial_sums = True
             m, k = x.shape
@@ -427,7 +447,9 @@ class HipOps:
             ):
                 return PendingLinear(x, weight, bias)
         if isinstance(x, (PendingNorm, PendingMerge)):
-            fused = self._linear_fused(x, weight, bias, out_dtype, kernel, swiglu, partial_sums, mfma_kernel, slices)
+            fused = None
+            if multiply is None:
+                fused = self._linear_fused(x, weight, bias, out_dtype, kernel, epilogue, partial_sums, mfma_kernel, slices)
             if fused is not None:
                 return fused
             x = self.settle(x)
@@ -449,6 +471,8 @@ class HipOps:
         if out_dtype not in (torch.float32, self.dtype):
             raise KernelError(f"linear output must be float32 or {self.dtype}")
         bias_f32 = int(bias is not None and bias.dtype == torch.float32)
+        if multiply is not None:
+            self._check(multiply, "multiplier", self.dtype, (m, n))
         if kernel == "auto" and self.dtype == torch.bfloat16 and k % 8 == 0:
             if slices is None:
                 slices = 1
@@ -464,18 +488,20 @@ class HipOps:
                 out_f32 = int(out_dtype == torch.float32)
             self._call(
                 "mlr_gemm_bf16", self._ptr(x), self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y), out_f32,
-                int(swiglu), slices, int(mfma_kernel), m, n, k, *scale, self._stream(),
+                epilogue, slices, int(mfma_kernel), m, n, k, *scale, self._ptr(multiply), self._stream(),
             )
             return y
         y = self._empty((m, n // 2 if swiglu else n), out_dtype)
         self._call(
             "mlr_gemm_simple", self._ptr(x), self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y),
-            int(out_dtype == torch.float32), int(swiglu), self.code, m, n, k, self._stream(),
+            int(out_dtype == torch.float32), epilogue, self.code, m, n, k, self._ptr(multiply), self._stream(),
         )
         return y
 
-    def _linear_fused(self, x, weight, bias, out_dtype, kernel, swiglu, partial_sums, mfma_kernel, slices):
-        """`linear` on a pending activation in one kernel, or None when that cannot be."""
+    def _linear_fused(self, x, weight, bias, out_dtype, kernel, epilogue, partial_sums, mfma_kernel, slices):
+        """`linear` on a pending activation in one kernel, or None when that cannot be.  `epilogue`:
+        the code of what happens to the sums (0 nothing, 1 the SwiGLU pairing, 2 and 3 activations)."""
+        swiglu = epilogue == 1
         m, k = x.shape
         if kernel != "auto" or mfma_kernel or self.dtype != torch.bfloat16 or k % 8 or m > self.FUSED_TOKENS:
             return None
@@ -497,11 +523,11 @@ class HipOps:
             y = self._empty((m, n // 2 if swiglu else n), out_dtype)
             self._call(
                 "mlr_gemm_norm_fused_bf16", *norm_args, self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y),
-                int(out_dtype == torch.float32), int(swiglu), 0, m, n, k, self._stream(),
+                int(out_dtype == torch.float32), epilogue, 0, m, n, k, self._stream(),
             )
             x.residual = residual
             return y
-        if swiglu or not self.tuning.fuse_merge or n * k * 2 > min(self.tuning.fuse_weight_bytes, (1 << 32) - 1):
+        if epilogue or not self.tuning.fuse_merge or n * k * 2 > min(self.tuning.fuse_weight_bytes, (1 << 32) - 1):
             return None
         if slices is None:
             slices = self.lib.mlr_gemm_bf16_slices(m, n, k, self.max_k_slices) if partial_sums else 1
@@ -752,8 +778,13 @@ class HipOps:
         kernel: str = "auto",
         defer_merge: bool = False,
         plan: Any = None,
+        chunk: Optional[int] = None,
     ):
         """Causal attention of the step's tokens over their requests' pages.
+
+        window / chunk: which of the keys 0..p a query at position p sees: with a window the last
+        `window` of them, with a chunked mask those from floor(p / chunk) * chunk on; at most one of
+        the two.
 
         defer_merge: the caller hands the result to `linear` and nothing else; when every
         entry has one token and their keys are cut into partitions, it may then receive a
@@ -784,6 +815,9 @@ class HipOps:
             raise KernelError("the block table is narrower than the longest context")
         if kernel not in ("auto", "fma"):
             raise KernelError("kernel must be 'auto' or 'fma'")
+        if chunk is not None and (chunk <= 0 or window):
+            raise KernelError("a chunked mask has a size > 0 and no window beside it")
+        chunk = int(chunk or 0)
         out = self._empty((tokens, num_heads * head_dim), self.dtype)
         width = block_table.shape[1]
         use_mfma = (
@@ -808,7 +842,7 @@ class HipOps:
                 "mlr_paged_attention_simple", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
                 self._ptr(block_table), width, self._ptr(ctx.token_entry), self._ptr(ctx.positions),
                 self._ptr(out), self.code, tokens, entries, num_heads, num_kv_heads, head_dim, block_size,
-                num_pages, float(scale), int(window or 0), self._stream(),
+                num_pages, float(scale), int(window or 0), chunk, self._stream(),
             )
             return out
         self._check(ctx.cu_q, "cu_q", torch.int32, (entries + 1,))
@@ -817,6 +851,8 @@ class HipOps:
             span = int(plan.max_decode_context)
             if window:
                 span = min(span, int(window) + 15)
+            if chunk:
+                span = min(span, chunk + 15)  # a partition starts at a multiple of 16 at or before the first key
             group_tiles = -(-(num_heads // num_kv_heads) // 16)
             base = num_decode * num_kv_heads * group_tiles
             part = max(64, self.decode_partition // 64 * 64)
@@ -830,13 +866,13 @@ class HipOps:
                 partial = self._empty((lib.mlr_attention_decode_scratch(entries, num_heads, splits),), torch.float32)
             leave_unmerged = (
                 defer_merge and self.tuning.fuse_merge and not num_tiles and num_decode == entries == tokens
-                and 1 < splits <= 64 and tokens <= self.FUSED_TOKENS
+                and 1 < splits <= 64 and tokens <= self.FUSED_TOKENS and not chunk
             )
             self._call(
                 "mlr_attention_decode", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
                 self._ptr(block_table), width, self._ptr(ctx.cu_q), self._ptr(ctx.context_lens), self._ptr(out),
                 self._ptr(partial), entries, num_heads, num_kv_heads, block_size, num_pages, float(scale),
-                int(window or 0), part, splits, int(not leave_unmerged), self._stream(), lib=lib,
+                int(window or 0), chunk, part, splits, int(not leave_unmerged), self._stream(), lib=lib,
             )
             if leave_unmerged:
                 return PendingMerge(
@@ -873,8 +909,83 @@ class HipOps:
                 "mlr_attention_prefill", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
                 self._ptr(block_table), width, self._ptr(tiles), num_tiles, wide, self._ptr(ctx.cu_q),
                 self._ptr(ctx.context_lens), self._ptr(out), num_heads, num_kv_heads, block_size, num_pages,
-                float(scale), int(window or 0), key_runs, self._ptr(partial), self._stream(), lib=lib,
+                float(scale), int(window or 0), chunk, key_runs, self._ptr(partial), self._stream(), lib=lib,
             )
+        return out
+
+    # ---- routed experts --------------------------------------------------------------------------------
+    def route_experts(
+        self, logits: torch.Tensor, correction: Optional[torch.Tensor], *, top: int, groups: int, keep_groups: int,
+        scale: float,
+    ) -> tuple[torch.Tensor, torch.Tensor]:
+        """Which experts every token uses (int32 [T, top]) and with what weight (float32 [T, top]),
+        from the router's float32 logits [T, experts]: sigmoid scores; the choice is made on score
+        + correction among the experts of the `keep_groups` best of `groups` groups of neighbours (a
+        group's score: the sum of its two largest); a chosen expert weighs its score times `scale`."""
+        self._check(logits, "router logits", torch.float32, (None, None))
+        tokens, experts = logits.shape
+        if correction is not None:
+            self._check(correction, "router correction", torch.float32, (experts,))
+        ids = self._empty((tokens, top), torch.int32)
+        weights = self._empty((tokens, top), torch.float32)
+        self._call(
+            "mlr_moe_route", self._ptr(logits), self._ptr(correction), self._ptr(ids), self._ptr(weights), tokens,
+            experts, int(top), int(groups), int(keep_groups), float(scale), self._stream(),
+        )
+        return ids, weights
+
+    def expert_products(
+        self,
+        h: torch.Tensor,
+        up_weight: torch.Tensor,
+        down_weight: torch.Tensor,
+        ids: torch.Tensor,
+        weights: torch.Tensor,
+        *,
+        experts: int,
+        activation: str,
+        kernel: str = "auto",
+    ) -> torch.Tensor:
+        """The chosen experts' outputs, weighted: float32 [top, T, hidden] with [j, t] = weights[t, j]
+        * down_e(act(up_e(h[t]))), e = ids[t, j]; the sum over j is the mixture's output, which a norm
+        adds to the stream in that order.  up_weight [experts * inner, hidden], down_weight [experts *
+        hidden, inner].  Three launches: the pairs sorted by expert into tiles of rows, and a grouped
+        product over the tiles for each of the two matrices (bfloat16 with hidden and inner multiples
+        of 8 on the matrix cores, everything else, and kernel="fma", as plain 32-bit arithmetic)."""
+        if kernel not in ("auto", "fma"):
+            raise KernelError("kernel must be 'auto' or 'fma'")
+        if activation not in ("relu2", "sigmoid"):
+            raise KernelError(f"unknown activation {activation!r}")
+        self._check(h, "expert input", self.dtype, (None, None))
+        tokens, hidden = h.shape
+        self._check(ids, "expert ids", torch.int32, (tokens, None))
+        top = ids.shape[1]
+        self._check(weights, "expert weights", torch.float32, (tokens, top))
+        if experts <= 0 or up_weight.shape[0] % experts:
+            raise KernelError("the stacked expert matrices do not divide by the number of experts")
+        inner = up_weight.shape[0] // experts
+        self._check(up_weight, "expert up weights", self.dtype, (experts * inner, hidden))
+        self._check(down_weight, "expert down weights", self.dtype, (experts * hidden, inner))
+        pairs = tokens * top
+        max_tiles = self.lib.mlr_moe_max_tiles(pairs, experts)
+        index = self._empty((pairs + experts + 1 + 2 * max_tiles,), torch.int32)
+        order, offsets, tiles = index[:pairs], index[pairs : pairs + experts + 1], index[pairs + experts + 1 :]
+        self._call(
+            "mlr_moe_align", self._ptr(ids), pairs, experts, max_tiles, self._ptr(order), self._ptr(offsets),
+            self._ptr(tiles), self._stream(),
+        )
+        mfma = int(kernel == "auto" and self.dtype == torch.bfloat16 and hidden % 8 == 0 and inner % 8 == 0)
+        act = self._empty((pairs, inner), self.dtype)
+        out = self._empty((top, tokens, hidden), torch.float32)
+        common = (self._ptr(order), self._ptr(offsets), self._ptr(tiles))
+        self._call(
+            "mlr_moe_gemm", self._ptr(h), self._ptr(up_weight), *common, _VP(None), self._ptr(act), 1, self.code, mfma,
+            max_tiles, tokens, top, inner, hidden, _EPILOGUES[activation], self._stream(),
+        )
+        self._call(
+            "mlr_moe_gemm", self._ptr(act), self._ptr(down_weight), *common, self._ptr(weights), self._ptr(out), 0,
+            self.code, mfma, max_tiles, tokens, top, hidden, inner, 0, self._stream(),
+        )
         return out
 
     # ---- sampling -----------------------------------------------------------------------------------

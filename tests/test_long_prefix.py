@@ -38,7 +38,7 @@ def _spying_ops(dtype, tuning):
 
         def _call(self, name, *args, lib=None):
             if name == "mlr_attention_prefill":
-                self.prefill_launches.append((int(args[8]), int(args[18])))
+                self.prefill_launches.append((int(args[8]), int(args[19])))
             return super()._call(name, *args, lib=lib)
 
     return SpyingOps(dtype, "cuda", tuning=tuning)
