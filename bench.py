@@ -38,6 +38,9 @@ around every call of an untimed extra step), and beside it what the vendor libra
 for the same shapes on the same card (torch's linear for the four products of a layer, its
 scaled_dot_product_attention for the attention): a yardstick for the hand-written kernels; none of
 those routines is on the engine's path.
+`designs`: the Fedolorn decoder (gated attention with a chunked mask, squared-ReLU or routed-expert
+feed-forward) beside the Qwen2 decoder at equal sizes (`DESIGN_POINTS`): decode steps of the engine at
+`--batch` and one prompt step, for each; `--design-points` picks some of them.
 `reference`: the reference's own published measurements, run here at their parameters with the
 0.5B shape (random weights and token ids of the published lengths; its figures are of an RTX 3060
 laptop GPU in float16 and stand beside for scale): the burst of 8 short requests under continuous and
@@ -96,7 +99,8 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--prompt-len", type=int, default=PROMPT_LEN)
     p.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
     p.add_argument("--seed", type=int, default=0)
-    p.add_argument("--workload", default="decode", choices=("decode", "burst", "chunked", "library", "reference"))
+    p.add_argument("--workload", default="decode", choices=("decode", "burst", "chunked", "library", "reference", "designs"))
+    p.add_argument("--design-points", default="", help="names of the `designs` workload's points to run, comma separated (default: all)")
     p.add_argument("--no-large", action="store_true", help="leave out the 7B and 32B points of the default run")
     p.add_argument("--samples", action="store_true", help="print every raw sample, not only their summary")
     p.add_argument("--layers-32b", type=int, default=None, help="layers of the 32B shape's points (default: all 64)")
@@ -606,7 +610,8 @@ def summary(samples_ms: list, keep: bool) -> dict:
 class Bench:
     """One model shape with random weights on the device, and the measurements on it."""
 
-    def __init__(self, args, name: str, layers, batches: list):
+    def __init__(self, args, name: str, layers, batches: list, data=None):
+        """`data`: a config.json content to use instead of the preset `name` (any registered architecture)."""
         import torch
 
         from mini_llm_runtime_amd.config.presets import load_preset
@@ -618,10 +623,16 @@ class Bench:
 
         self.args = args
         self.name = name
-        data = load_preset(name)
-        self.full_layers = int(data["num_hidden_layers"])
-        if layers is not None:
-            data["num_hidden_layers"] = int(layers)
+        if data is None:
+            data = load_preset(name)
+        if "num_hidden_layers" in data:
+            self.full_layers = int(data["num_hidden_layers"])
+            if layers is not None:
+                data["num_hidden_layers"] = int(layers)
+        else:  # a configuration that lists its layers
+            self.full_layers = len(data["layers"])
+            if layers is not None:
+                data = dict(data, layers=list(data["layers"])[: int(layers)])
         self.config = config_from_dict(data)
         self.dtype = parse_dtype(args.dtype)
         self.short = "bf16" if self.dtype == torch.bfloat16 else "fp32"
@@ -641,7 +652,7 @@ class Bench:
     def prompt(self) -> list:
         import torch
 
-        return torch.randint(0, self.config.vocab_size, (self.args.prompt_len,), generator=self.gen).tolist()
+        return torch.randint(0, self.model.spec.vocab_size, (self.args.prompt_len,), generator=self.gen).tolist()
 
     def sync(self) -> None:
         import torch
@@ -701,9 +712,9 @@ class Bench:
 
     def decode_bytes(self, batch: int, mean_context: float) -> tuple:
         """Bytes a decode step has to read: every weight it uses once, and the live requests' cache."""
-        model, config = self.model, self.config
+        model = self.model
         weight_bytes = model.weight_bytes()
-        if not config.tie_word_embeddings:  # an untied input table is only gathered from
+        if not model.spec.tie_word_embeddings:  # an untied input table is only gathered from
             weight_bytes -= model.embed_weight.numel() * model.embed_weight.element_size()
         return weight_bytes, weight_bytes + batch * mean_context * self.kv_bytes_per_token()
 
@@ -744,17 +755,7 @@ class Bench:
             self.cache.release_request(rid)
         host, dev = host[1:], dev[1:]
         ms = sorted(host)[len(host) // 2]
-        d = config.head_dim
-        per_layer = (
-            config.hidden_size * (config.num_attention_heads + 2 * config.num_key_value_heads) * d
-            + config.num_attention_heads * d * config.hidden_size
-            + 3 * config.hidden_size * config.intermediate_size
-        )
-        flops = (
-            2 * tokens * per_layer * config.num_hidden_layers
-            + config.num_hidden_layers * config.num_attention_heads * 4 * d * tokens * (tokens + 1) // 2
-            + 2 * config.vocab_size * config.hidden_size
-        )
+        flops = self.prefill_flops(tokens)
         return {
             "value": round(tokens * 1e3 / ms, 1),
             "tokens": tokens,
@@ -763,6 +764,35 @@ class Bench:
             "ms_device": round(sorted(dev)[len(dev) // 2], 3),
             "samples_ms": [round(x, 3) for x in host],
         }
+
+    def prefill_flops(self, tokens: int) -> int:
+        """Multiply-adds times two of one prompt of `tokens` tokens (the head for one row)."""
+        config = self.config
+        if hasattr(config, "num_attention_heads"):
+            d = config.head_dim
+            per_layer = (
+                config.hidden_size * (config.num_attention_heads + 2 * config.num_key_value_heads) * d
+                + config.num_attention_heads * d * config.hidden_size
+                + 3 * config.hidden_size * config.intermediate_size
+            )
+            return (
+                2 * tokens * per_layer * config.num_hidden_layers
+                + config.num_hidden_layers * config.num_attention_heads * 4 * d * tokens * (tokens + 1) // 2
+                + 2 * config.vocab_size * config.hidden_size
+            )
+        # a configuration that lists its layers (attention with a gate and a chunked mask; dense or routed
+        # feed-forward, of which a token uses `top` experts and the router)
+        width, flops = config.width, 2 * config.vocab * config.width
+        for layer in config.layers:
+            a, m = layer.mixer, layer.mlp
+            per_token = width * (a.heads * a.dim + a.kv_heads * (a.dim + a.vdim) + 2 * a.heads * a.vdim)
+            if m is not None:
+                per_token += 2 * width * m.ff * (m.top if m.kind == "moe" else 1) + (width * m.experts if m.kind == "moe" else 0)
+            chunk = a.mask_size or tokens
+            whole, rest = divmod(tokens, chunk)
+            pairs = whole * chunk * (chunk + 1) // 2 + rest * (rest + 1) // 2  # (query, visible key) pairs
+            flops += 2 * tokens * per_token + 2 * a.heads * (a.dim + a.vdim) * pairs
+        return flops
 
     def peak_memory(self) -> dict:
         """Device memory in GiB: the most this process's tensors held at one time since the shape was
@@ -791,6 +821,85 @@ class Bench:
         for name in ("runner", "cache", "model", "sampler"):
             setattr(self, name, None)
         self.collect()
+
+
+# The `designs` workload: the Fedolorn decoder beside the Qwen2 decoder at equal sizes.  Equal means: the
+# same width, heads, head size, layers and vocabulary, and a feed-forward with the same number of weights a
+# token uses: Qwen2's SwiGLU has three matrices of `inter` features, a squared-ReLU feed-forward two of
+# 1.5 x inter, and `top` experts of `ff` features are two matrices of top x ff.  The chunk is longer than
+# the context, so both attend over the same keys.
+DESIGN_POINTS = {
+    # name: (width, heads, kv heads, head size, SwiGLU inter, layers run, Fedolorn feed-forward)
+    "dense-0.5b": (896, 14, 2, 64, 4864, 12, {"kind": "dense", "ff": 7296}),
+    "dense-7b": (3584, 28, 4, 128, 18944, 4, {"kind": "dense", "ff": 28416}),
+    "moe-2048x64e": (2048, 16, 4, 128, 3072, 8, {
+        "kind": "moe", "expert": {"ff": 768},
+        "router": {"experts": 64, "top": 6, "scale": 2.5, "groups": {"count": 8, "keep": 4}},
+    }),
+    "moe-4096x128e": (4096, 32, 8, 128, 8192, 4, {
+        "kind": "moe", "expert": {"ff": 1536},
+        "router": {"experts": 128, "top": 8, "scale": 2.5, "groups": {"count": 8, "keep": 4}},
+    }),
+}
+DESIGN_VOCAB = 32768
+
+
+def design_configs(name: str) -> dict:
+    width, heads, kv_heads, dim, inter, layers, mlp = DESIGN_POINTS[name]
+    fedolorn = {
+        "architecture": "Fedolorn", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-5},
+        "embedding": {"scale": 1.0},
+        "layers": [
+            {"type": "attention", "mlp": mlp,
+             "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim**-0.5, "mask": {"size": 8192}}}
+            for _ in range(layers)
+        ],
+    }
+    qwen2 = {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "vocab_size": DESIGN_VOCAB, "hidden_size": width,
+        "intermediate_size": inter, "num_hidden_layers": layers, "num_attention_heads": heads,
+        "num_key_value_heads": kv_heads, "head_dim": dim, "max_position_embeddings": 32768, "rms_norm_eps": 1e-5,
+        "rope_theta": 1000000.0, "hidden_act": "silu", "tie_word_embeddings": True,
+    }
+    return {"fedolorn": fedolorn, "qwen2": qwen2}
+
+
+def design_comparison(args) -> dict:
+    """Prefill of one prompt and decode steps of the engine at `--batch` for each point and both designs."""
+    names = [n for n in args.design_points.split(",") if n.strip()] or list(DESIGN_POINTS)
+    points = {}
+    for name in names:
+        point = {}
+        for design, data in design_configs(name).items():
+            bench = Bench(args, f"{name}/{design}", None, [args.batch], data=data)
+            run = bench.decode(args.batch, args.warmup, args.steps)
+            weight_bytes, _ = bench.decode_bytes(args.batch, 0)
+            prefill = bench.prefill()
+            point[design] = {
+                "decode_tokens_per_s": round(args.batch * 1e3 / run["ms"], 1),
+                "decode_ms_per_step": round(run["ms"], 4),
+                "prefill_tokens_per_s": prefill["value"],
+                "prefill_ms": prefill["ms"],
+                "prefill_frac_of_peak": prefill["frac"],
+                "weight_bytes": int(weight_bytes),
+                "layers": len(bench.model.layers),
+            }
+            bench.close()
+            print(f"# {name} {design}: {point[design]}", file=sys.stderr, flush=True)
+        point["decode_ratio"] = round(point["fedolorn"]["decode_tokens_per_s"] / point["qwen2"]["decode_tokens_per_s"], 3)
+        point["prefill_ratio"] = round(point["fedolorn"]["prefill_tokens_per_s"] / point["qwen2"]["prefill_tokens_per_s"], 3)
+        points[name] = point
+    return {
+        "metric": "decode and prefill tokens/s of two designs at equal sizes",
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic (random weights made on the device, uniform random token ids)",
+        "config": {"global_batch": args.batch, "prompt_len": args.prompt_len, "vocab": DESIGN_VOCAB, "kv_block_size": BLOCK_SIZE},
+        "points": points,
+    }
 
 
 def large_point(args, name: str, layers, batches=(8,), workload: str = "") -> dict:
@@ -854,6 +963,12 @@ def main() -> int:
 
     sys.path.insert(0, str(Path(__file__).resolve().parent))
     import mini_llm_runtime_amd  # noqa: F401
+
+    if args.workload == "designs":
+        line = design_comparison(args)
+        line["env"] = environment()
+        print(json.dumps(line), flush=True)
+        return 0
 
     batches = [args.batch] + [int(b) for b in args.points.split(",") if b.strip()]
     bench = Bench(args, args.config, args.layers, batches)
