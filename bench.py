@@ -100,6 +100,7 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
     p.add_argument("--seed", type=int, default=0)
     p.add_argument("--workload", default="decode", choices=("decode", "burst", "chunked", "library", "reference", "designs"))
+    p.add_argument("--design-only", default="", choices=("", "fedolorn", "qwen2"), help="run one of the two designs of the `designs` workload (for profiles)")
     p.add_argument("--design-points", default="", help="names of the `designs` workload's points to run, comma separated (default: all)")
     p.add_argument("--no-large", action="store_true", help="leave out the 7B and 32B points of the default run")
     p.add_argument("--samples", action="store_true", help="print every raw sample, not only their summary")
@@ -871,6 +872,8 @@ def design_comparison(args) -> dict:
     for name in names:
         point = {}
         for design, data in design_configs(name).items():
+            if args.design_only and design != args.design_only:
+                continue
             bench = Bench(args, f"{name}/{design}", None, [args.batch], data=data)
             run = bench.decode(args.batch, args.warmup, args.steps)
             weight_bytes, _ = bench.decode_bytes(args.batch, 0)
@@ -886,8 +889,9 @@ def design_comparison(args) -> dict:
             }
             bench.close()
             print(f"# {name} {design}: {point[design]}", file=sys.stderr, flush=True)
-        point["decode_ratio"] = round(point["fedolorn"]["decode_tokens_per_s"] / point["qwen2"]["decode_tokens_per_s"], 3)
-        point["prefill_ratio"] = round(point["fedolorn"]["prefill_tokens_per_s"] / point["qwen2"]["prefill_tokens_per_s"], 3)
+        if len(point) == 2:
+            point["decode_ratio"] = round(point["fedolorn"]["decode_tokens_per_s"] / point["qwen2"]["decode_tokens_per_s"], 3)
+            point["prefill_ratio"] = round(point["fedolorn"]["prefill_tokens_per_s"] / point["qwen2"]["prefill_tokens_per_s"], 3)
         points[name] = point
     return {
         "metric": "decode and prefill tokens/s of two designs at equal sizes",

@@ -109,6 +109,10 @@ __device__ __forceinline__ void row_scales_finish(const GemmEpilogue& ep, const 
 __device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
 
 // Store four consecutive output features n..n+3 of token m (n is a multiple of 4).
+// ACTIVATIONS false leaves the element-wise activations and the multiplier out: for the one kernel
+// whose accumulators fill the register file (the 256 x 320 tile), where the longer epilogue made the
+// compiler keep them in memory, ten times slower; the host never sends such a product there.
+template <bool ACTIVATIONS = true>
 __device__ __forceinline__ void store4(const GemmEpilogue& ep, int64_t m, int n, int N, float v0, float v1,
                                        float v2, float v3) {
   float v[4] = {v0, v1, v2, v3};
@@ -134,21 +138,23 @@ __device__ __forceinline__ void store4(const GemmEpilogue& ep, int64_t m, int n,
       if (n + i < N) v[i] += load_as_f32(ep.bias, n + i, ep.bias_is_f32);
   }
   const int64_t at = m * N + n;
-  if (ep.swiglu == kEpRelu2) {
+  if constexpr (ACTIVATIONS) {
+    if (ep.swiglu == kEpRelu2) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float r = fmaxf(v[i], 0.f);
-      v[i] = r * r;
+      for (int i = 0; i < 4; ++i) {
+        const float r = fmaxf(v[i], 0.f);
+        v[i] = r * r;
+      }
+    } else if (ep.swiglu == kEpSigmoid) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = 1.0f / (1.0f + __expf(-v[i]));
     }
-  } else if (ep.swiglu == kEpSigmoid) {
+    if (ep.multiply != nullptr) {
+      const bf16* other = static_cast<const bf16*>(ep.multiply) + at;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = 1.0f / (1.0f + __expf(-v[i]));
-  }
-  if (ep.multiply != nullptr) {
-    const bf16* other = static_cast<const bf16*>(ep.multiply) + at;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (n + i < N) v[i] *= to_f32(other[i]);
+      for (int i = 0; i < 4; ++i)
+        if (n + i < N) v[i] *= to_f32(other[i]);
+    }
   }
   if (ep.out_is_f32) {
     float* y = static_cast<float*>(ep.y) + at;
@@ -175,11 +181,12 @@ __device__ __forceinline__ void store4(const GemmEpilogue& ep, int64_t m, int n,
 
 // Store one accumulator tile (4 consecutive features of one token per lane): the
 // final result, or this K slice's partial sums.
+template <bool ACTIVATIONS = true>
 __device__ __forceinline__ void finish4(const GemmEpilogue& ep, int slice, int slices, int m, int n, int M, int N,
                                         const float (&v)[4]) {
   if (m >= M || n >= N) return;
   if (slices == 1) {
-    store4(ep, m, n, N, v[0], v[1], v[2], v[3]);
+    store4<ACTIVATIONS>(ep, m, n, N, v[0], v[1], v[2], v[3]);
     return;
   }
   const int64_t at = (static_cast<int64_t>(slice) * M + m) * N + n;

@@ -734,7 +734,7 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
         const int n = n0 + (wn * WN + i) * 32 + g * 8 + h * 4;
         const float v[4] = {acc[i][j][g * 4 + 0] * scale, acc[i][j][g * 4 + 1] * scale, acc[i][j][g * 4 + 2] * scale,
                             acc[i][j][g * 4 + 3] * scale};
-        finish4(ep, slice, slices, m, n, M, N, v);
+        finish4<(WM * WN < 10)>(ep, slice, slices, m, n, M, N, v);  // ten blocks a wavefront: the registers are full
       }
     }
 }
@@ -1151,6 +1151,8 @@ int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f3
               "sums of squares come with their number per row (1..65536) and an eps >= 0");
   GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu, row_sumsq, sumsq_parts, norm_eps, multiply};
   if (kernel == 0) kernel = choose_kernel(m, n, k, slices);
+  // the 256 x 320 tile has no room for the activations and the multiplier in its epilogue
+  if (kernel == 48 && (swiglu >= kEpRelu2 || multiply != nullptr)) kernel = 45;
   if (gemm_bf16(static_cast<const bf16*>(x), static_cast<const bf16*>(w), ep, m, n, k, slices, kernel, stream) != 0)
     return -1;
   MLR_LAUNCH_CHECK();

@@ -156,6 +156,10 @@ def is_current(module: Module, folder: Optional[Path] = None) -> bool:
 RESOURCE_REMARKS = "-Rpass-analysis=kernel-resource-usage"
 _KERNEL_NAME = re.compile(r"remark: Function Name: (\S+)")
 _KERNEL_SPILL = re.compile(r"remark:\s+VGPRs Spill: (\d+)")
+# Arrays that the compiler could not keep in registers (an epilogue loop it stopped unrolling, and the
+# accumulators it indexes, once went there) are not counted as spills but as scratch memory per lane:
+# the same ten times slower, so they count the same, in registers of four bytes.
+_KERNEL_SCRATCH = re.compile(r"remark:\s+ScratchSize \[bytes/lane\]: (\d+)")
 _SOURCE_CONTEXT = re.compile(r"^\s*\d*\s*\|")
 
 
@@ -179,6 +183,9 @@ def _run(cmd: Sequence[str], what: str) -> dict[str, int]:
         spilled = _KERNEL_SPILL.search(line)
         if spilled and kernel is not None:
             spills[kernel] = max(spills[kernel], int(spilled.group(1)))
+        scratch = _KERNEL_SCRATCH.search(line)
+        if scratch and kernel is not None:
+            spills[kernel] = max(spills[kernel], int(scratch.group(1)) // 4)
         if "[-Rpass-analysis=kernel-resource-usage]" in line:
             in_report = True  # the source line and the caret under it belong to the report
             continue
