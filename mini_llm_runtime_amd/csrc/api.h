@@ -192,16 +192,18 @@ int mlr_moe_route(const float* logits, const float* correction, int* ids, float*
                   int top, int groups, int keep, float scale, hipStream_t stream);
 // The (token, choice) pairs p = token * top + choice sorted by expert: sorted [pairs], offsets
 // [experts + 1], tiles [max_tiles, 2] = (expert, first row of `sorted`) with up to
-// mlr_moe_tile_rows() rows each, unused tiles (-1, 0).  max_tiles >= mlr_moe_max_tiles(pairs, experts).
-int mlr_moe_tile_rows();
-int mlr_moe_max_tiles(int pairs, int experts);
-int mlr_moe_align(const int* ids, int pairs, int experts, int max_tiles, int* sorted, int* offsets, int* tiles,
-                  hipStream_t stream);
+// mlr_moe_tile_rows(big) rows each (16, or 64 with `big`), unused tiles (-1, 0).  max_tiles >=
+// mlr_moe_max_tiles(pairs, experts, big).
+int mlr_moe_tile_rows(int big);
+int mlr_moe_max_tiles(int pairs, int experts, int big);
+int mlr_moe_align(const int* ids, int pairs, int experts, int big, int max_tiles, int* sorted, int* offsets,
+                  int* tiles, hipStream_t stream);
 // One grouped product over those tiles; w is [experts, n, k] in `dtype` (0 float32, 1 bfloat16).
 // up 1: a = h [tokens, k]; out [pairs, n] in `dtype`, row r = act(h[sorted[r] / top] w[e]^T), act 0
 // none, 2 squared ReLU, 3 sigmoid.  up 0: a = the rows of the first product [pairs, k]; out float32
-// [top, tokens, n], out[choice, token] = pair_weights[p] * (a[r] w[e]^T).  mfma 1: on the matrix
-// cores (bfloat16, k % 8 == 0), else plain 32-bit FMA arithmetic.
+// [top, tokens, n], out[choice, token] = pair_weights[p] * (a[r] w[e]^T).  mfma 1 and 2: on the matrix
+// cores (bfloat16, k % 8 == 0; 1 streams tiles of 16 rows, 2 runs tiles of 64 rows through LDS and
+// needs n % 8 == 0), 0: plain 32-bit FMA arithmetic (tiles of 16 rows).
 int mlr_moe_gemm(const void* a, const void* w, const int* sorted, const int* offsets, const int* tiles,
                  const float* pair_weights, void* out, int up, int dtype, int mfma, int max_tiles, int tokens, int top,
                  int n, int k, int act, hipStream_t stream);

@@ -235,13 +235,17 @@ __global__ __launch_bounds__(256) void moe_gemm_simple_kernel(const T* __restric
 
 // ---- grouped products in bfloat16 on the matrix cores ---------------------------------------------
 //
-// The same two products.  A workgroup of four wavefronts owns 16 rows of a tile (the columns of the
-// 16 x 16 x 32 block; weights are the row operand, as in the other product kernels) and 64 features,
-// 16 per wavefront.  A lane reads 8 consecutive k of one weight row and of one input row per block:
-// both operands straight from memory, no LDS; rows past the tile's end and features past N read
-// nothing and multiply zeros.  Few rows a tile (decoding) make this a streaming kernel, whose time
-// is the expert weights it reads; with many rows a tile the weights are re-read by every 16 rows
-// from L2.
+// The same two products, two kernels.
+//
+// Streaming (tiles of 16 rows; decoding, where an expert sees a few rows): a workgroup of four
+// wavefronts owns 16 rows of a tile (the columns of the 16 x 16 x 32 block; weights are the row
+// operand, as in the other product kernels) and 64 features, 16 per wavefront.  A lane reads 8
+// consecutive k of one weight row and of one input row per block, both straight from memory through
+// range-checked buffer loads (rows past the tile's end, features past N and k past K read zeros, no
+// branch around a load), eight blocks in flight before the first product: the kernel's time is the
+// expert weights it streams, read once (non-temporal).
+constexpr int kMoeDepth = 8;
+
 template <bool UP>
 __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w,
                                                             const int* __restrict__ sorted,
@@ -249,37 +253,41 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16* __restri
                                                             const int* __restrict__ tiles,
                                                             const float* __restrict__ pair_weights,
                                                             void* __restrict__ out, int tokens, int top, int N, int K,
-                                                            int act) {
+                                                            int act, int a_rows) {
   const int expert = tiles[2 * blockIdx.x];
   if (expert < 0) return;
   const int row0 = tiles[2 * blockIdx.x + 1];
   const int row_end = offsets[expert + 1];
   const int lane = threadIdx.x % kWave;
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int col = lane % 16;   // operand row: weight row / input row of the tile
   const int quad = lane / 16;  // which 8 of a block's 32 k
-  const int n_base = blockIdx.y * 64 + wave * 16;
+  const int n_base = (blockIdx.y * (blockDim.x / kWave) + wave) * 16;  // 16 features a wavefront
   if (n_base >= N) return;
   // the input row this lane loads (as the column operand), and the rows whose sums it ends up with
   const int in_row = row0 + col;
   const int in_pair = in_row < row_end ? sorted[in_row] : -1;
-  const bf16* arow = nullptr;
-  if (in_pair >= 0) arow = UP ? a + static_cast<int64_t>(in_pair / top) * K : a + static_cast<int64_t>(in_row) * K;
+  const int a_row = in_pair < 0 ? -1 : (UP ? in_pair / top : in_row);
+  const unsigned row_bytes = static_cast<unsigned>(K) * 2u;
+  const __amdgpu_buffer_rsrc_t wbuf =
+      make_buffer(w + static_cast<int64_t>(expert) * N * K, static_cast<unsigned>(N) * row_bytes);
+  const __amdgpu_buffer_rsrc_t abuf = make_buffer(a, static_cast<unsigned>(a_rows) * row_bytes);
   const int wn = n_base + col;
-  const bf16* wrow = wn < N ? w + (static_cast<int64_t>(expert) * N + wn) * K : nullptr;
+  const unsigned w_off = wn < N ? static_cast<unsigned>(wn) * row_bytes : kOutOfBuffer;
+  const unsigned a_off = a_row >= 0 ? static_cast<unsigned>(a_row) * row_bytes : kOutOfBuffer;
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-  const bf16x8_t zero = zero_bf16x8();
-  // two blocks of 32 k a turn; the loop's bounds are the same for every lane
-  for (int kb = 0; kb < K; kb += 64) {
-    const int k1 = kb + quad * 8;
-    const int k2 = k1 + 32;
-    bf16x8_t wa = zero, xa = zero, wb = zero, xb = zero;
-    if (wrow != nullptr && k1 < K) wa = load_bf16x8(wrow + k1);
-    if (arow != nullptr && k1 < K) xa = load_bf16x8(arow + k1);
-    if (wrow != nullptr && k2 < K) wb = load_bf16x8(wrow + k2);
-    if (arow != nullptr && k2 < K) xb = load_bf16x8(arow + k2);
-    acc = mfma_16x16x32(wa, xa, acc);
-    acc = mfma_16x16x32(wb, xb, acc);
+  for (int kb = 0; kb < K; kb += 32 * kMoeDepth) {
+    bf16x8_t wv[kMoeDepth], xv[kMoeDepth];
+#pragma unroll
+    for (int u = 0; u < kMoeDepth; ++u) {
+      const int k = kb + u * 32 + quad * 8;
+      const unsigned koff = static_cast<unsigned>(k) * 2u;
+      const bool in = k < K;
+      wv[u] = buffer_load_bf16x8_once(wbuf, in && w_off != kOutOfBuffer ? w_off + koff : kOutOfBuffer);
+      xv[u] = buffer_load_bf16x8(abuf, in && a_off != kOutOfBuffer ? a_off + koff : kOutOfBuffer);
+    }
+#pragma unroll
+    for (int u = 0; u < kMoeDepth; ++u) acc = mfma_16x16x32(wv[u], xv[u], acc);
   }
   // acc[i]: feature n_base + quad * 4 + i of tile row `col`
   if (in_pair < 0) return;
@@ -308,6 +316,178 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16* __restri
   }
 }
 
+// Tiled (prompts, where an expert sees hundreds of rows): a workgroup owns a tile of 64 x RB rows and
+// 128 features; k in slices of 64 through two LDS buffers (rows padded to 144 bytes: free of bank
+// conflicts for the operand pattern of the 32 x 32 x 16 block), the next slice on its way into
+// registers while this one is multiplied.  Wavefront (wr, wc) of 2 x 2 owns rows wr * 32 RB .. + 32 RB
+// and features wc * 64 .. + 64: 2 RB blocks of 32 x 32; with RB = 2 every operand read from LDS serves
+// two products.
+constexpr int kBigCols = 128;
+constexpr int kBigK = 64;
+constexpr int kBigLd = kBigK + 8;  // bf16 elements per LDS row
+constexpr int big_rows(int rb) { return 64 * rb; }
+constexpr int big_lds_bytes(int rb) { return 2 * (kBigCols + big_rows(rb)) * kBigLd * 2 + big_rows(rb) * 4; }
+
+template <bool UP, int RB>
+__global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w,
+                                                             const int* __restrict__ sorted,
+                                                             const int* __restrict__ offsets,
+                                                             const int* __restrict__ tiles,
+                                                             const float* __restrict__ pair_weights,
+                                                             void* __restrict__ out, int tokens, int top, int N, int K,
+                                                             int act, int a_rows) {
+  constexpr int kRows = big_rows(RB);
+  const int expert = tiles[2 * blockIdx.x];
+  if (expert < 0) return;
+  const int row0 = tiles[2 * blockIdx.x + 1];
+  const int row_end = offsets[expert + 1];
+  extern __shared__ __attribute__((aligned(16))) unsigned char moe_lds[];
+  bf16* const ws = reinterpret_cast<bf16*>(moe_lds);   // [2][kBigCols][kBigLd]
+  bf16* const xs = ws + 2 * kBigCols * kBigLd;         // [2][kRows][kBigLd]
+  int* const pair_of = reinterpret_cast<int*>(xs + 2 * kRows * kBigLd);  // [kRows]
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wr = wave / 2;
+  const int wc = wave % 2;
+  const int n0 = blockIdx.y * kBigCols;
+  if (tid < kRows) pair_of[tid] = row0 + tid < row_end ? sorted[row0 + tid] : -1;
+  __syncthreads();
+  const unsigned row_bytes = static_cast<unsigned>(K) * 2u;
+  const __amdgpu_buffer_rsrc_t wbuf =
+      make_buffer(w + static_cast<int64_t>(expert) * N * K, static_cast<unsigned>(N) * row_bytes);
+  const __amdgpu_buffer_rsrc_t abuf = make_buffer(a, static_cast<unsigned>(a_rows) * row_bytes);
+  // what this thread moves per slice: 16-byte pieces of the weight tile and of the input tile
+  // (piece c: row c / 8, k piece c % 8), the same rows for every slice
+  constexpr int kWPieces = kBigCols * 8 / 256;
+  constexpr int kXPieces = kRows * 8 / 256;
+  unsigned w_off[kWPieces], x_off[kXPieces];
+  const int piece = tid % 8;  // the same for all of a thread's pieces: 256 is a multiple of 8
+#pragma unroll
+  for (int i = 0; i < kWPieces; ++i) {
+    const int row = (tid + i * 256) / 8;
+    w_off[i] = n0 + row < N ? static_cast<unsigned>(n0 + row) * row_bytes + piece * 16u : kOutOfBuffer;
+  }
+#pragma unroll
+  for (int i = 0; i < kXPieces; ++i) {
+    const int row = (tid + i * 256) / 8;
+    const int pair = pair_of[row];
+    const int src = pair < 0 ? -1 : (UP ? pair / top : row0 + row);
+    x_off[i] = src >= 0 ? static_cast<unsigned>(src) * row_bytes + piece * 16u : kOutOfBuffer;
+  }
+  const int lds_at = (tid / 8) * kBigLd + piece * 8;  // piece i of either tile: + i * 32 rows
+  bf16x8_t wreg[kWPieces], xreg[kXPieces];
+  auto fetch = [&](int k0) {
+    const bool k_in = k0 + piece * 8 < K;
+    const unsigned koff = static_cast<unsigned>(k0) * 2u;
+#pragma unroll
+    for (int i = 0; i < kWPieces; ++i)
+      wreg[i] = buffer_load_bf16x8(wbuf, k_in && w_off[i] != kOutOfBuffer ? w_off[i] + koff : kOutOfBuffer);
+#pragma unroll
+    for (int i = 0; i < kXPieces; ++i)
+      xreg[i] = buffer_load_bf16x8(abuf, k_in && x_off[i] != kOutOfBuffer ? x_off[i] + koff : kOutOfBuffer);
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < kWPieces; ++i)
+      *reinterpret_cast<bf16x8_t*>(ws + buf * kBigCols * kBigLd + lds_at + i * 32 * kBigLd) = wreg[i];
+#pragma unroll
+    for (int i = 0; i < kXPieces; ++i)
+      *reinterpret_cast<bf16x8_t*>(xs + buf * kRows * kBigLd + lds_at + i * 32 * kBigLd) = xreg[i];
+  };
+  f32x16_t acc[RB][2];
+#pragma unroll
+  for (int r = 0; r < RB; ++r)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[r][b][i] = 0.f;
+  const int r32 = lane % 32;
+  const int khalf = lane / 32;  // which 8 of a block's 16 k
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = 0; k0 < K; k0 += kBigK) {
+    const bool more = k0 + kBigK < K;
+    if (more) fetch(k0 + kBigK);
+    const bf16* wt = ws + buf * kBigCols * kBigLd + (wc * 64 + r32) * kBigLd + khalf * 8;
+    const bf16* xt = xs + buf * kRows * kBigLd + (wr * 32 * RB + r32) * kBigLd + khalf * 8;
+#pragma unroll
+    for (int ks = 0; ks < kBigK / 16; ++ks) {
+      const bf16x8_t w0 = *reinterpret_cast<const bf16x8_t*>(wt + ks * 16);
+      const bf16x8_t w1 = *reinterpret_cast<const bf16x8_t*>(wt + 32 * kBigLd + ks * 16);
+#pragma unroll
+      for (int r = 0; r < RB; ++r) {
+        const bf16x8_t xb = *reinterpret_cast<const bf16x8_t*>(xt + r * 32 * kBigLd + ks * 16);
+        acc[r][0] = mfma_32x32x16(w0, xb, acc[r][0]);
+        acc[r][1] = mfma_32x32x16(w1, xb, acc[r][1]);
+      }
+    }
+    if (more) stage(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+  // acc[r][b][i]: feature n0 + wc * 64 + b * 32 + (i / 4) * 8 + khalf * 4 + i % 4 of tile row
+  // wr * 32 RB + r * 32 + r32
+#pragma unroll
+  for (int r = 0; r < RB; ++r) {
+    const int row = wr * 32 * RB + r * 32 + r32;
+    const int pair = pair_of[row];
+    if (pair < 0) continue;
+    const int token = pair / top;
+    const int choice = pair - token * top;
+    const float pw = UP ? 1.f : pair_weights[pair];
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n0 + wc * 64 + b * 32 + g * 8 + khalf * 4;
+        if (n >= N) continue;  // N is a multiple of 8 here: four features are all inside or all outside
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = acc[r][b][g * 4 + i];
+        if (UP) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if (act == 2) {
+              v[i] = fmaxf(v[i], 0.f);
+              v[i] *= v[i];
+            } else if (act == 3) {
+              v[i] = 1.0f / (1.0f + __expf(-v[i]));
+            }
+          }
+          const u16x4_t packed = {f32_to_bf16(v[0]).bits, f32_to_bf16(v[1]).bits, f32_to_bf16(v[2]).bits,
+                                  f32_to_bf16(v[3]).bits};
+          *reinterpret_cast<u16x4_t*>(static_cast<bf16*>(out) + static_cast<int64_t>(row0 + row) * N + n) = packed;
+        } else {
+          float* dst = static_cast<float*>(out) + (static_cast<int64_t>(choice) * tokens + token) * N + n;
+          *reinterpret_cast<f32x4_t*>(dst) = f32x4_t{pw * v[0], pw * v[1], pw * v[2], pw * v[3]};
+        }
+      }
+  }
+}
+
+template <bool UP, int RB>
+static int launch_moe_tiled(const bf16* a, const bf16* w, const int* sorted, const int* offsets, const int* tiles,
+                            const float* pair_weights, void* out, int max_tiles, int tokens, int top, int n, int k,
+                            int act, int a_rows, hipStream_t stream) {
+  static bool configured = false;
+  if (!configured) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(moe_gemm_tiled_kernel<UP, RB>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, big_lds_bytes(RB));
+    if (e != hipSuccess) {
+      set_error(std::string("mlr_moe_gemm: cannot raise the LDS limit: ") + hipGetErrorString(e));
+      return -1;
+    }
+    configured = true;
+  }
+  const dim3 grid(max_tiles, (n + kBigCols - 1) / kBigCols);
+  moe_gemm_tiled_kernel<UP, RB><<<grid, 256, big_lds_bytes(RB), stream>>>(a, w, sorted, offsets, tiles, pair_weights, out,
+                                                                        tokens, top, n, k, act, a_rows);
+  return 0;
+}
+
 }  // namespace mlr
 
 using namespace mlr;
@@ -327,29 +507,32 @@ int mlr_moe_route(const float* logits, const float* correction, int* ids, float*
   return 0;
 }
 
-// Rows of one tile of the grouped products (fixed by their kernels).
-int mlr_moe_tile_rows() { return kMoeRows; }
+// Rows of one tile of the grouped products: `big` 0 the kernels for few rows an expert (16), 1 and 2
+// the tiled matrix-core kernel for many (64 and 128).
+int mlr_moe_tile_rows(int big) { return big ? big_rows(big) : kMoeRows; }
 
 // The most tiles `pairs` pairs over `experts` experts can make.
-int mlr_moe_max_tiles(int pairs, int experts) {
-  const int most = pairs / kMoeRows + experts;  // full tiles, and at most one that is not per expert
+int mlr_moe_max_tiles(int pairs, int experts, int big) {
+  const int most = pairs / mlr_moe_tile_rows(big) + experts;  // full tiles, and at most one that is not per expert
   return most < pairs ? most : pairs;
 }
 
-int mlr_moe_align(const int* ids, int pairs, int experts, int max_tiles, int* sorted, int* offsets, int* tiles,
+int mlr_moe_align(const int* ids, int pairs, int experts, int big, int max_tiles, int* sorted, int* offsets, int* tiles,
                   hipStream_t stream) {
   MLR_REQUIRE(ids && sorted && offsets && tiles, "null pointer");
-  MLR_REQUIRE(pairs > 0 && experts > 0 && experts <= 4096 && max_tiles > 0, "bad sizes");
-  MLR_REQUIRE(max_tiles >= mlr_moe_max_tiles(pairs, experts), "too few tiles for these pairs");
-  moe_align_kernel<<<1, 1024, 2 * static_cast<size_t>(experts) * sizeof(int), stream>>>(ids, pairs, experts, kMoeRows,
-                                                                                      max_tiles, sorted, offsets, tiles);
+  MLR_REQUIRE(pairs > 0 && experts > 0 && experts <= 4096 && max_tiles > 0 && big >= 0 && big <= 2, "bad sizes");
+  MLR_REQUIRE(max_tiles >= mlr_moe_max_tiles(pairs, experts, big), "too few tiles for these pairs");
+  moe_align_kernel<<<1, 1024, 2 * static_cast<size_t>(experts) * sizeof(int), stream>>>(
+      ids, pairs, experts, mlr_moe_tile_rows(big), max_tiles, sorted, offsets, tiles);
   MLR_LAUNCH_CHECK();
   return 0;
 }
 
 // One of the two grouped products (`up` 1: act = f(h w_up^T) for the sorted rows, `act` 0 none, 2
 // squared ReLU, 3 sigmoid; `up` 0: out[choice, token] = weight * (act w_down^T), float32).  a and w
-// in `dtype`; w is [experts, n, k].  `mfma` 1: the matrix-core kernel (bfloat16, k % 8 == 0).
+// in `dtype`; w is [experts, n, k].  `mfma` 1: the streaming matrix-core kernel (bfloat16, k % 8 == 0;
+// tiles of 16 rows), 2 and 3: the tiled one (tiles of 64 and of 128 rows, as mlr_moe_align made them
+// with `big` 1 and 2; n % 8 == 0 too); 0: plain arithmetic (tiles of 16 rows).
 int mlr_moe_gemm(const void* a, const void* w, const int* sorted, const int* offsets, const int* tiles,
                  const float* pair_weights, void* out, int up, int dtype, int mfma, int max_tiles, int tokens, int top,
                  int n, int k, int act, hipStream_t stream) {
@@ -361,15 +544,38 @@ int mlr_moe_gemm(const void* a, const void* w, const int* sorted, const int* off
   MLR_REQUIRE((n + kMoeCols - 1) / kMoeCols <= 65535, "too many features for one launch");
   const dim3 grid(max_tiles, (n + kMoeCols - 1) / kMoeCols);
   if (mfma) {
-    MLR_REQUIRE(dtype == kBF16 && k % 8 == 0, "the matrix-core kernel takes bfloat16 and k % 8 == 0");
-    MLR_REQUIRE(reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
-                "a and w must be 16-byte aligned");
-    if (up)
-      moe_gemm_mfma_kernel<true><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(a), static_cast<const bf16*>(w),
-                                                           sorted, offsets, tiles, pair_weights, out, tokens, top, n, k, act);
-    else
-      moe_gemm_mfma_kernel<false><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(a), static_cast<const bf16*>(w),
-                                                            sorted, offsets, tiles, pair_weights, out, tokens, top, n, k, act);
+    MLR_REQUIRE(mfma >= 1 && mfma <= 3, "mfma must be within 0..3");
+    MLR_REQUIRE(dtype == kBF16 && k % 8 == 0, "the matrix-core kernels take bfloat16 and k % 8 == 0");
+    MLR_REQUIRE(mfma == 1 || n % 8 == 0, "the tiled kernel needs n % 8 == 0");
+    MLR_REQUIRE(reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(out) % 16 == 0,
+                "a, w and out must be 16-byte aligned");
+    // rows of `a`: the tokens for the first product, the pairs for the second; both fit 32-bit offsets
+    const int64_t a_rows = up ? tokens : static_cast<int64_t>(tokens) * top;
+    MLR_REQUIRE(a_rows * k * 2 < (1ll << 32) && static_cast<int64_t>(n) * k * 2 < (1ll << 31),
+                "the inputs or one expert's matrix are too large for 32-bit offsets");
+    const bf16* ab = static_cast<const bf16*>(a);
+    const bf16* wb = static_cast<const bf16*>(w);
+    const int rows = static_cast<int>(a_rows);
+    if (mfma >= 2) {
+      int status;
+      if (mfma == 2)
+        status = up ? launch_moe_tiled<true, 1>(ab, wb, sorted, offsets, tiles, pair_weights, out, max_tiles, tokens, top, n, k, act, rows, stream)
+                    : launch_moe_tiled<false, 1>(ab, wb, sorted, offsets, tiles, pair_weights, out, max_tiles, tokens, top, n, k, act, rows, stream);
+      else
+        status = up ? launch_moe_tiled<true, 2>(ab, wb, sorted, offsets, tiles, pair_weights, out, max_tiles, tokens, top, n, k, act, rows, stream)
+                    : launch_moe_tiled<false, 2>(ab, wb, sorted, offsets, tiles, pair_weights, out, max_tiles, tokens, top, n, k, act, rows, stream);
+      if (status != 0) return -1;
+    } else {
+      // four wavefronts (64 features) a workgroup, or two where that leaves the compute units with too
+      // few workgroups to keep their loads in flight
+      const int waves = static_cast<int64_t>(max_tiles) * ((n + 63) / 64) < 2048 ? 2 : 4;
+      const dim3 small_grid(max_tiles, (n + waves * 16 - 1) / (waves * 16));
+      if (up)
+        moe_gemm_mfma_kernel<true><<<small_grid, waves * kWave, 0, stream>>>(ab, wb, sorted, offsets, tiles, pair_weights, out, tokens, top, n, k, act, rows);
+      else
+        moe_gemm_mfma_kernel<false><<<small_grid, waves * kWave, 0, stream>>>(ab, wb, sorted, offsets, tiles, pair_weights, out, tokens, top, n, k, act, rows);
+    }
     MLR_LAUNCH_CHECK();
     return 0;
   }

@@ -40,9 +40,9 @@ _SIGNATURES = {
     "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP], _I),
     "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _I, _VP, _I, _F, _VP, _VP], _I),
     "mlr_moe_route": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _VP], _I),
-    "mlr_moe_tile_rows": ([], _I),
-    "mlr_moe_max_tiles": ([_I, _I], _I),
-    "mlr_moe_align": ([_VP, _I, _I, _I, _VP, _VP, _VP, _VP], _I),
+    "mlr_moe_tile_rows": ([_I], _I),
+    "mlr_moe_max_tiles": ([_I, _I, _I], _I),
+    "mlr_moe_align": ([_VP, _I, _I, _I, _I, _VP, _VP, _VP, _VP], _I),
     "mlr_moe_gemm": ([_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_residual_parts": ([_I, _I], _I),
     "mlr_gemm_residual_bf16": ([_VP, _VP, _VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _VP], _I),
@@ -967,14 +967,21 @@ class HipOps:
         self._check(up_weight, "expert up weights", self.dtype, (experts * inner, hidden))
         self._check(down_weight, "expert down weights", self.dtype, (experts * hidden, inner))
         pairs = tokens * top
-        max_tiles = self.lib.mlr_moe_max_tiles(pairs, experts)
+        mfma = int(kernel == "auto" and self.dtype == torch.bfloat16 and hidden % 8 == 0 and inner % 8 == 0)
+        # many rows an expert (on average: the host does not know the routing): tiles of 64 rows through
+        # LDS; few: tiles of 16 rows that stream the expert's weights
+        big = int(bool(mfma) and pairs >= self.tuning.moe_tiled_rows * experts)
+        if big and pairs >= self.tuning.moe_wide_tiled_rows * experts:
+            big = 2  # tiles of 128 rows
+        if big:
+            mfma = 1 + big
+        max_tiles = self.lib.mlr_moe_max_tiles(pairs, experts, big)
         index = self._empty((pairs + experts + 1 + 2 * max_tiles,), torch.int32)
         order, offsets, tiles = index[:pairs], index[pairs : pairs + experts + 1], index[pairs + experts + 1 :]
         self._call(
-            "mlr_moe_align", self._ptr(ids), pairs, experts, max_tiles, self._ptr(order), self._ptr(offsets),
+            "mlr_moe_align", self._ptr(ids), pairs, experts, big, max_tiles, self._ptr(order), self._ptr(offsets),
             self._ptr(tiles), self._stream(),
         )
-        mfma = int(kernel == "auto" and self.dtype == torch.bfloat16 and hidden % 8 == 0 and inner % 8 == 0)
         act = self._empty((pairs, inner), self.dtype)
         out = self._empty((top, tokens, hidden), torch.float32)
         common = (self._ptr(order), self._ptr(offsets), self._ptr(tiles))

@@ -52,8 +52,13 @@ class KernelTuning:
     # features of ONE token, so the float32 stream is read and written 16 bytes at a time at a stride of
     # a row, where the norm kernel reads whole rows.)
 
+    # Routed experts: from this many (token, choice) pairs per expert on (on average) the grouped products
+    # run in tiles of 64 rows through LDS; below, in tiles of 16 rows that stream the weights.
+    moe_tiled_rows: int = 32
+    moe_wide_tiled_rows: int = 96  # and from this many on in tiles of 128 rows
+
     def __post_init__(self) -> None:
-        for name in ("decode_partition", "decode_max_groups", "max_k_slices", "wide_attention_groups", "key_run_groups", "fuse_weight_bytes",
+        for name in ("moe_tiled_rows", "moe_wide_tiled_rows", "decode_partition", "decode_max_groups", "max_k_slices", "wide_attention_groups", "key_run_groups", "fuse_weight_bytes",
                      "finish_weight_bytes", "finish_activation_bytes", "finish_min_tokens",
                      "finish_max_tokens"):
             value = getattr(self, name)
