@@ -445,3 +445,65 @@ def test_greedy_generation_through_the_engine(tmp_path, which, backend, dtype):
                 assert float(logits[best] - logits[tok]) < 3e-2 * float(logits.abs().max())
                 break
             seq.append(tok)
+
+
+# ---- the command line and the replay program --------------------------------------------------------------
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def test_preset_and_random_model_writer(tmp_path):
+    from helpers import read_weights
+    from mini_llm_runtime_amd import cli
+    from mini_llm_runtime_amd.config.presets import preset_names
+
+    assert "fedolorn-tiny" in preset_names()
+    assert cli.main(["random-model", "--config", "fedolorn-tiny", "--seed", "2", "--out", str(tmp_path / "m")]) == 0
+    cfg, w = read_weights(tmp_path / "m")
+    assert cfg["architecture"] == "Fedolorn" and w["embed"].shape == (384, 96)
+    assert w["l1.mlp.e7.down"].shape == (96, 48) and w["l1.mlp.correction"].shape == (8,) and "l2.norm2" not in w
+    assert float(w["l0.norm1"].float().abs().max()) < 0.5  # stored around zero
+    plain.forward(cfg, w, [1, 2, 3])  # the plain implementation reads the same folder
+
+
+@pytest.mark.gpu
+def test_generate_command_and_trace_replay(tmp_path, gpu_device):
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    folder, cfg, weights = make_dir(tmp_path, "P")
+    prompt = random_tokens(21, cfg["vocab"], 4)
+    proc = subprocess.run(
+        [sys.executable, "-m", "mini_llm_runtime_amd.cli", "generate", "--model", str(folder), "--dtype", "float32",
+         "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "5"],
+        cwd=ROOT, capture_output=True, text=True, timeout=300,
+    )
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    out = json.loads(proc.stdout.strip().splitlines()[-1])
+    seq = list(prompt)
+    for tok in out["generated_token_ids"]:
+        assert tok == int(torch.argmax(plain.forward(cfg, weights, seq)[-1]))
+        seq.append(tok)
+    # the replay program: two requests in portions beside each other, slots and pages used again
+    toks = {"a": random_tokens(40, cfg["vocab"], 5), "b": random_tokens(27, cfg["vocab"], 6), "c": random_tokens(33, cfg["vocab"], 7)}
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": toks["a"][:25], "want": [0, 24]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": toks["a"][25:27], "want": [1]}, {"id": "b", "tokens": toks["b"], "want": [26]}], "end": ["b"]},
+        {"step": 2, "entries": [{"id": "a", "tokens": toks["a"][27:], "want": [12]}, {"id": "c", "tokens": toks["c"][:32], "want": []}], "end": ["a"]},
+        {"step": 3, "entries": [{"id": "c", "tokens": toks["c"][32:], "want": [0]}], "end": ["c"]},
+    ]
+    proc = subprocess.run(
+        [str(ROOT / "bin" / "trace_run"), "--model", str(folder), "--dtype", "bfloat16", "--out", str(tmp_path / "o"),
+         "--max-tokens", "128", "--max-live", "2"],
+        input="".join(json.dumps(s) + "\n" for s in steps), cwd=ROOT, capture_output=True, text=True, timeout=300,
+    )
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+    wanted = {0: [("a", 0), ("a", 24)], 1: [("a", 26), ("b", 26)], 2: [("a", 39)], 3: [("c", 32)]}
+    for step, rows in wanted.items():
+        got = torch.from_numpy(np.fromfile(tmp_path / "o" / f"{step}.f32", dtype="<f4").reshape(len(rows), cfg["vocab"]))
+        for row, (rid, pos) in zip(got, rows):
+            ref = plain.forward(cfg, weights, toks[rid][: pos + 1])[-1]
+            assert float((row.double() - ref).pow(2).sum().sqrt() / ref.pow(2).sum().sqrt()) < 6e-2, (step, rid, pos)
