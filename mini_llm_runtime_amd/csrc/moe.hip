@@ -316,6 +316,127 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16* __restri
   }
 }
 
+// Streaming through LDS (tiles of 16 rows, as above): the same work with loads that cover whole lines.
+// A workgroup owns 16 rows of a tile and 64 features; k in slices of 128.  Sixteen neighbouring lanes
+// fetch the 256 contiguous bytes that a slice holds of one weight row (the kernel above reads 64 bytes
+// of 16 different rows per instruction, which streams a large matrix at little more than half the
+// rate), two slices ahead in registers, and stage them through two LDS buffers whose rows of 288 bytes
+// are free of bank conflicts for the operand pattern of the 16 x 16 x 32 block.  Wavefront w multiplies
+// features w * 16 .. + 16.
+constexpr int kStCols = 64;
+constexpr int kStK = 128;
+constexpr int kStLd = kStK + 16;  // bf16 elements per LDS row: 288 bytes
+
+template <bool UP>
+__global__ __launch_bounds__(256) void moe_gemm_stream_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w,
+                                                              const int* __restrict__ sorted,
+                                                              const int* __restrict__ offsets,
+                                                              const int* __restrict__ tiles,
+                                                              const float* __restrict__ pair_weights,
+                                                              void* __restrict__ out, int tokens, int top, int N, int K,
+                                                              int act, int a_rows) {
+  const int expert = tiles[2 * blockIdx.x];
+  if (expert < 0) return;
+  const int row0 = tiles[2 * blockIdx.x + 1];
+  const int row_end = offsets[expert + 1];
+  __shared__ __attribute__((aligned(16))) bf16 ws[2][kStCols * kStLd];
+  __shared__ __attribute__((aligned(16))) bf16 xs[2][kMoeRows * kStLd];
+  __shared__ int pair_of[kMoeRows];
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int n0 = blockIdx.y * kStCols;
+  if (tid < kMoeRows) pair_of[tid] = row0 + tid < row_end ? sorted[row0 + tid] : -1;
+  __syncthreads();
+  const unsigned row_bytes = static_cast<unsigned>(K) * 2u;
+  const __amdgpu_buffer_rsrc_t wbuf =
+      make_buffer(w + static_cast<int64_t>(expert) * N * K, static_cast<unsigned>(N) * row_bytes);
+  const __amdgpu_buffer_rsrc_t abuf = make_buffer(a, static_cast<unsigned>(a_rows) * row_bytes);
+  // per slice a thread moves four 16-byte pieces of the weight tile (rows prow, prow + 16, ...) and one
+  // of the input tile (row prow), all at k piece `piece` of the slice
+  const int piece = tid % 16;
+  const int prow = tid / 16;
+  unsigned w_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = n0 + prow + i * 16;
+    w_off[i] = row < N ? static_cast<unsigned>(row) * row_bytes + piece * 16u : kOutOfBuffer;
+  }
+  const int my_pair = pair_of[prow];
+  const int src = my_pair < 0 ? -1 : (UP ? my_pair / top : row0 + prow);
+  const unsigned x_off = src >= 0 ? static_cast<unsigned>(src) * row_bytes + piece * 16u : kOutOfBuffer;
+  const int lds_at = prow * kStLd + piece * 8;
+  bf16x8_t w_a[4], w_b[4], x_a, x_b;  // two slices on their way
+  auto fetch = [&](bf16x8_t(&wreg)[4], bf16x8_t& xreg, int k0) {
+    const bool k_in = k0 + piece * 8 < K;
+    const unsigned koff = static_cast<unsigned>(k0) * 2u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      wreg[i] = buffer_load_bf16x8_once(wbuf, k_in && w_off[i] != kOutOfBuffer ? w_off[i] + koff : kOutOfBuffer);
+    xreg = buffer_load_bf16x8(abuf, k_in && x_off != kOutOfBuffer ? x_off + koff : kOutOfBuffer);
+  };
+  auto stage = [&](const bf16x8_t(&wreg)[4], const bf16x8_t& xreg, int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8_t*>(&ws[buf][lds_at + i * 16 * kStLd]) = wreg[i];
+    *reinterpret_cast<bf16x8_t*>(&xs[buf][lds_at]) = xreg;
+  };
+  const int col = lane % 16;
+  const int quad = lane / 16;
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  auto multiply = [&](int buf) {
+    const bf16* wt = &ws[buf][(wave * 16 + col) * kStLd + quad * 8];
+    const bf16* xt = &xs[buf][col * kStLd + quad * 8];
+#pragma unroll
+    for (int ks = 0; ks < kStK / 32; ++ks)
+      acc = mfma_16x16x32(*reinterpret_cast<const bf16x8_t*>(wt + ks * 32),
+                          *reinterpret_cast<const bf16x8_t*>(xt + ks * 32), acc);
+  };
+  const int slices = (K + kStK - 1) / kStK;
+  fetch(w_a, x_a, 0);
+  if (slices > 1) fetch(w_b, x_b, kStK);
+  stage(w_a, x_a, 0);
+  __syncthreads();
+  // two slices a turn, so that the register sets and the LDS buffers keep their names; `slices` is the
+  // same for every thread, so are the barriers
+  for (int s = 0; s < slices; s += 2) {
+    if (s + 2 < slices) fetch(w_a, x_a, (s + 2) * kStK);
+    multiply(0);
+    if (s + 1 < slices) stage(w_b, x_b, 1);
+    __syncthreads();
+    if (s + 1 >= slices) break;
+    if (s + 3 < slices) fetch(w_b, x_b, (s + 3) * kStK);
+    multiply(1);
+    if (s + 2 < slices) stage(w_a, x_a, 0);
+    __syncthreads();
+  }
+  // acc[i]: feature n0 + wave * 16 + quad * 4 + i of tile row `col`
+  const int pair = pair_of[col];
+  if (pair < 0) return;
+  const int token = pair / top;
+  const int choice = pair - token * top;
+  const int n = n0 + wave * 16 + quad * 4;
+  if (UP) {
+    bf16* dst = static_cast<bf16*>(out) + static_cast<int64_t>(row0 + col) * N + n;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float v = acc[i];
+      if (act == 2) {
+        v = fmaxf(v, 0.f);
+        v *= v;
+      } else if (act == 3) {
+        v = 1.0f / (1.0f + __expf(-v));
+      }
+      if (n + i < N) dst[i] = f32_to_bf16(v);
+    }
+  } else {
+    const float pw = pair_weights[pair];
+    float* dst = static_cast<float*>(out) + (static_cast<int64_t>(choice) * tokens + token) * N + n;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n + i < N) dst[i] = pw * acc[i];
+  }
+}
+
 // Tiled (prompts, where an expert sees hundreds of rows): a workgroup owns a tile of 64 x RB rows and
 // 128 features; k in slices of 64 through two LDS buffers (rows padded to 144 bytes: free of bank
 // conflicts for the operand pattern of the 32 x 32 x 16 block), the next slice on its way into
@@ -566,6 +687,13 @@ int mlr_moe_gemm(const void* a, const void* w, const int* sorted, const int* off
         status = up ? launch_moe_tiled<true, 2>(ab, wb, sorted, offsets, tiles, pair_weights, out, max_tiles, tokens, top, n, k, act, rows, stream)
                     : launch_moe_tiled<false, 2>(ab, wb, sorted, offsets, tiles, pair_weights, out, max_tiles, tokens, top, n, k, act, rows, stream);
       if (status != 0) return -1;
+    } else if (static_cast<int64_t>(n) * k * 2 >= (1ll << 20)) {
+      // an expert's matrix of a megabyte or more: whole lines through LDS
+      const dim3 stream_grid(max_tiles, (n + kStCols - 1) / kStCols);
+      if (up)
+        moe_gemm_stream_kernel<true><<<stream_grid, 256, 0, stream>>>(ab, wb, sorted, offsets, tiles, pair_weights, out, tokens, top, n, k, act, rows);
+      else
+        moe_gemm_stream_kernel<false><<<stream_grid, 256, 0, stream>>>(ab, wb, sorted, offsets, tiles, pair_weights, out, tokens, top, n, k, act, rows);
     } else {
       // four wavefronts (64 features) a workgroup, or two where that leaves the compute units with too
       // few workgroups to keep their loads in flight

@@ -88,9 +88,18 @@ CONFIGS = {
         (_attention(4, 2, 32, 32, 0.35, 20), None),
         (_attention(2, 1, 48, 16, 0.3, 33), None),
     ]),
+    # long requests: hundreds of keys in a chunk (the decode kernel's partitions and their merge, several
+    # key tiles of the prompt kernel), a chunk edge deep inside a prompt and passed while decoding
+    "U": _model(200, 128, 1e-5, 1.0, [
+        (_attention(4, 2, 64, 64, 0.15, 320), _moe(8, 2, 32, 1.2, (2, 1))),
+        (_attention(2, 1, 64, 32, 0.15, 512), None),
+    ]),
 }
-BLOCK = {"P": 16, "Q": 8, "R": 4, "S": 16, "T": 8}
-LENGTHS = {"P": (1, 9, 50, 83, 37, 64), "Q": (2, 19, 35, 66, 45), "R": (3, 30, 41, 58), "S": (5, 17, 140, 70, 97), "T": (1, 24, 75, 41, 130)}
+BLOCK = {"P": 16, "Q": 8, "R": 4, "S": 16, "T": 8, "U": 16}
+LENGTHS = {
+    "P": (1, 9, 50, 83, 37, 64), "Q": (2, 19, 35, 66, 45), "R": (3, 30, 41, 58), "S": (5, 17, 140, 70, 97),
+    "T": (1, 24, 75, 41, 130), "U": (660, 341),
+}
 
 
 def make_weights(cfg: dict, seed: int) -> dict[str, torch.Tensor]:
@@ -341,8 +350,10 @@ def _needle_model(mask: int, dim: int, vdim: int) -> tuple[dict, dict]:
 
 
 @pytest.mark.parametrize("backend,dtype", CASES)
-@pytest.mark.parametrize("mask,dim,vdim", [(16, 16, 16), (37, 32, 16), (64, 16, 48), (5, 24, 24)])
+@pytest.mark.parametrize("mask,dim,vdim", [(16, 16, 16), (37, 32, 16), (64, 16, 48), (5, 24, 24), (300, 64, 64)])
 def test_one_key_just_inside_and_just_outside_the_chunk(tmp_path, backend, dtype, mask, dim, vdim):
+    if backend == "double" and mask > 100:
+        pytest.skip("the CPU stand-in is slow at this length")
     cfg, weights = _needle_model(mask, dim, vdim)
     folder = Path(tmp_path) / "needle"
     folder.mkdir()
@@ -386,8 +397,8 @@ FAMILIES = {
 @pytest.mark.parametrize("family", list(FAMILIES))
 @pytest.mark.parametrize("which", list(CONFIGS))
 def test_schedule_matches_plain(tmp_path, which, family, backend, dtype):
-    if backend == "double" and which in ("S",) and family != "mixed":
-        pytest.skip("the CPU stand-in is slow at this size; the mixed schedule covers it")
+    if backend == "double" and (which == "U" or (which == "S" and family != "mixed")):
+        pytest.skip("the CPU stand-in is slow at this size")
     folder, cfg, weights = make_dir(tmp_path, which)
     requests = _requests(which)
     steps = FAMILIES[family](requests)
