@@ -300,7 +300,7 @@ def test_routing_kernel(experts, top, groups, keep):
 
 
 @pytest.mark.parametrize("dtype", GPU_CASES)
-@pytest.mark.parametrize("tokens,hidden,inner,experts,top", [(1, 64, 40, 8, 2), (7, 72, 20, 6, 1), (50, 100, 36, 4, 4), (200, 128, 64, 16, 4), (19, 64, 24, 5, 3), (300, 64, 40, 4, 2), (130, 200, 136, 3, 1)])
+@pytest.mark.parametrize("tokens,hidden,inner,experts,top", [(1, 64, 40, 8, 2), (7, 72, 20, 6, 1), (50, 100, 36, 4, 4), (200, 128, 64, 16, 4), (19, 64, 24, 5, 3), (300, 64, 40, 4, 2), (130, 200, 136, 3, 1), (9, 1024, 512, 4, 2), (21, 1032, 520, 3, 2)])
 def test_grouped_expert_products(dtype, tokens, hidden, inner, experts, top):
     ops = _ops("hip", dtype)
     g = torch.Generator().manual_seed(tokens + experts)
