@@ -835,11 +835,11 @@ DESIGN_POINTS = {
     "dense-7b": (3584, 28, 4, 128, 18944, 4, {"kind": "dense", "ff": 28416}),
     "moe-2048x64e": (2048, 16, 4, 128, 3072, 8, {
         "kind": "moe", "expert": {"ff": 768},
-        "router": {"experts": 64, "top": 6, "scale": 2.5, "groups": {"count": 8, "keep": 4}},
+        "router": {"experts": 64, "top": 6, "scale": 2.0, "groups": {"count": 8, "keep": 4}},
     }),
     "moe-4096x128e": (4096, 32, 8, 128, 8192, 4, {
         "kind": "moe", "expert": {"ff": 1536},
-        "router": {"experts": 128, "top": 8, "scale": 2.5, "groups": {"count": 8, "keep": 4}},
+        "router": {"experts": 128, "top": 8, "scale": 2.0, "groups": {"count": 8, "keep": 4}},
     }),
 }
 DESIGN_VOCAB = 32768

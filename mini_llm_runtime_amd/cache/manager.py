@@ -78,19 +78,17 @@ class KVGroup:
 
     def dead_blocks(self, num_tokens: int) -> int:
         """How many leading pages no query at position >= num_tokens can see."""
-        if self.spec.window is None:
-            return 0
-        first_visible = num_tokens - self.spec.window + 1
-        return max(0, first_visible // self.block_size)
+        return max(0, self.spec.first_live_position(num_tokens) // self.block_size)
 
     def lifetime_blocks(self, max_tokens: int, max_step_tokens: int) -> int:
         """Most pages a request holds at one time over its life."""
         full = blocks_for(max_tokens, self.block_size)
-        if self.spec.window is None:
+        span = self.spec.live_span()
+        if span is None:
             return full
-        # the window before the first query of a step, the step's own tokens, and
-        # one page for the misalignment of the window's start
-        bounded = blocks_for(self.spec.window - 1 + max_step_tokens, self.block_size) + 1
+        # what the first query of a step may still see (a window, the run of a chunked mask), the
+        # step's own tokens, and one page for the misalignment of the first live position
+        bounded = blocks_for(span + max_step_tokens, self.block_size) + 1
         return min(full, bounded)
 
     def storage_bytes(self) -> int:

@@ -41,9 +41,29 @@ class PagedSpec(SiteCacheSpec):
 
     window: None keeps every token; an integer W keeps only what a query may still see, the W most
     recent positions including its own, so pages that every later query has passed are given back.
+    chunk: an integer C likewise keeps only the run of C positions (runs counted from position 0)
+    that the next query lies in: a query never sees beyond the start of its own run.
+    The manager asks `first_live_position` and `live_span`, never which of the two it is.
     """
 
     window: Optional[int] = None
+    chunk: Optional[int] = None
+
+    def first_live_position(self, num_tokens: int) -> int:
+        """The first position that a query at position >= num_tokens may still see."""
+        if self.window is not None:
+            return max(0, num_tokens - self.window + 1)
+        if self.chunk is not None:
+            return num_tokens - num_tokens % self.chunk
+        return 0
+
+    def live_span(self) -> Optional[int]:
+        """Most positions before a step's first query that the step may see (None: all of them)."""
+        if self.window is not None:
+            return self.window - 1
+        if self.chunk is not None:
+            return self.chunk - 1
+        return None
 
     def attach(self, manager: Any, site: int) -> None:
         manager.add_paged_site(site, self)
@@ -100,12 +120,15 @@ class PagedKVSpec(PagedSpec):
     head_dim: int
     window: Optional[int] = None
     value_head_dim: Optional[int] = None
+    chunk: Optional[int] = None
 
     def __post_init__(self) -> None:
         if self.num_kv_heads <= 0 or self.head_dim <= 0:
             raise ValueError("PagedKVSpec sizes must be > 0")
         if self.window is not None and self.window <= 0:
             raise ValueError("PagedKVSpec.window must be > 0 or None")
+        if self.chunk is not None and (self.chunk <= 0 or self.window is not None):
+            raise ValueError("PagedKVSpec.chunk must be > 0 or None, and comes without a window")
         if self.value_head_dim is not None and self.value_head_dim < 0:
             raise ValueError("PagedKVSpec.value_head_dim must be >= 0 or None")
 

@@ -589,8 +589,8 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   // Loads are unconditional (a page that is absent or past the end reads page 0 instead) so
   // that the tile loop stays free of branches.  Keys read that way need no clearing: their
   // scores are masked by position.  Values are cleared, since 0 * NaN would reach the output;
-  // that can only happen in the last tile and under a window, whose early pages may be gone (a
-  // chunked mask gives no page back: what lies before a query's chunk was written by its own request).
+  // that can only happen in the last tile, under a window, whose early pages may be gone, and in the
+  // tile that a chunk starts in, whose positions before the chunk may lie in pages given back.
   // The page ids of a tile are looked up one tile ahead of its loads (two ahead of its use):
   // a lookup right before the loads that need it would put two trips to memory, one after the
   // other, into every turn of the loop.
@@ -614,7 +614,7 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
       if (!in) bad = bad || (k_row[i] < lim && kt0 + k_row[i] >= k_begin_raw);
       t.k[i] = load_bf16x8(key_pages + (static_cast<uint64_t>(in ? static_cast<uint32_t>(page) : 0u) * page_elems + k_in_page[i]));
     }
-    const bool guard = lim < kTileK || window > 0;  // uniform
+    const bool guard = lim < kTileK || window > 0 || (chunk > 0 && kt0 < k_begin_raw);  // uniform
 #pragma unroll
     for (int i = 0; i < kPieces; ++i) {
       const int page = v_ids[i];

@@ -36,7 +36,8 @@ class GQAAttention(Mixer):
     Options that other decoders use:
     chunk: instead of all earlier keys (or the last `window`), a query at position p sees the keys
         of its own run of `chunk` positions only: floor(p / chunk) * chunk .. p.  Runs are counted
-        from position 0 of the request, whatever portions its prompt is processed in.
+        from position 0 of the request, whatever portions its prompt is processed in.  The pages of
+        runs that every later query has left behind are given back, as under a window.
     value_dim: value heads of another width than query and key heads.  The kernels and the pages
         know one head size, so when the two differ all heads are laid out at one common size D
         (the larger, rounded up to a multiple of 16) with zero rows in the projections: zeros add
@@ -161,7 +162,7 @@ class GQAAttention(Mixer):
         return {"position": self.position} if self.position is not None else {}
 
     def cache_spec(self) -> PagedKVSpec:
-        return PagedKVSpec(self.num_kv_heads, self.kernel_dim, self.window)
+        return PagedKVSpec(self.num_kv_heads, self.kernel_dim, self.window, chunk=self.chunk)
 
     def plan(self, ops, shape: PlanInput) -> Optional[MixerPlan]:
         make = getattr(ops, "attention_plan", None)  # the kernel library knows what its kernels want

@@ -79,7 +79,7 @@ CONFIGS = {
     ]),
     # matrix-core sizes: head size 64 with a group of four, 128 against 64, sixteen experts
     "S": _model(512, 128, 1e-5, 2.0, [
-        (_attention(4, 1, 64, 64, 0.125, 32), _moe(16, 4, 64, 2.5, (4, 2))),
+        (_attention(4, 1, 64, 64, 0.14, 32), _moe(16, 4, 64, 2.2, (4, 2))),
         (_attention(2, 2, 128, 64, 0.09, 48), _dense(256)),
         (_attention(8, 4, 32, 32, 0.18, 16), _moe(16, 3, 32, 1.5, (8, 3))),
     ]),
@@ -518,3 +518,64 @@ def test_generate_command_and_trace_replay(tmp_path, gpu_device):
         for row, (rid, pos) in zip(got, rows):
             ref = plain.forward(cfg, weights, toks[rid][: pos + 1])[-1]
             assert float((row.double() - ref).pow(2).sum().sqrt() / ref.pow(2).sum().sqrt()) < 6e-2, (step, rid, pos)
+
+
+# ---- pages of runs that every later query has left behind ------------------------------------------------
+
+def test_chunked_sites_give_pages_back():
+    from mini_llm_runtime_amd.cache import PagedKVSpec
+    from mini_llm_runtime_amd.cache.manager import CacheManager
+
+    spec = PagedKVSpec(2, 16, chunk=8)
+    assert [spec.first_live_position(n) for n in (0, 7, 8, 15, 16, 23)] == [0, 0, 8, 8, 16, 16] and spec.live_span() == 7
+    with pytest.raises(ValueError):
+        PagedKVSpec(2, 16, window=4, chunk=8)
+    cache = CacheManager([spec], block_size=4, num_blocks=8, max_requests=2, dtype=torch.float32, device=torch.device("cpu"))
+    assert cache.lifetime_blocks(1000, 6) == [blocks(7 + 6, 4) + 1]
+    request = cache.create_request("a")
+    fed = 0
+    for n in (5, 6, 6, 6, 3):  # 26 tokens through a pool that holds whole requests of 32 at most
+        cache.begin_step([("a", n)])
+        passed = cache.commit_step()
+        fed += n
+        live = [b for b in request.tables[0] if b >= 0]
+        assert len(live) == blocks(fed, 4) - (fed - fed % 8) // 4
+        cache.check_invariants()
+        if fed >= 8:
+            assert all(b == -1 for b in request.tables[0][: (fed - fed % 8) // 4])
+    assert passed == {"a": {0: passed["a"][0]}} and len(passed["a"][0]) == 2  # 24 tokens behind: the run 16..23 went
+    cache.release_request("a")
+    assert cache.groups[0].allocator.free_count == 8
+
+
+def blocks(tokens: int, size: int) -> int:
+    return -(-tokens // size)
+
+
+CONFIGS["V"] = _model(160, 64, 1e-6, 1.2, [
+    (_attention(4, 2, 16, 16, 0.3, 16), _dense(80)),
+    (_attention(2, 2, 32, 32, 0.2, 16), None),
+])
+
+
+@pytest.mark.parametrize("backend,dtype", CASES)
+def test_generation_in_a_pool_smaller_than_a_request(tmp_path, backend, dtype):
+    """A chunked model's request needs the pages of one run and of a step, not of its whole length: 75
+    tokens (19 pages of 4) go through a pool of 9 pages, whose pages are used again and again."""
+    folder, cfg, weights = make_dir(tmp_path, "V")
+    ops = _ops(backend, dtype)
+    engine = ContinuousBatchEngine.from_model_dir(
+        folder, dtype=ops.dtype, ops=ops, block_size=4, num_blocks=9, max_running_requests=1, max_batch_tokens=8,
+    )
+    prompt = random_tokens(45, cfg["vocab"], 3)
+    tokens = engine.generate([prompt], max_new_tokens=30)[0]
+    assert len(tokens) == 30
+    seq = list(prompt)
+    for i, tok in enumerate(tokens):
+        logits = plain.forward(cfg, weights, seq)[-1]
+        best = int(torch.argmax(logits))
+        if tok != best:
+            assert dtype == torch.bfloat16, f"token {i}: {tok} != {best}"
+            assert float(logits[best] - logits[tok]) < 3e-2 * float(logits.abs().max())
+            break
+        seq.append(tok)
