@@ -20,6 +20,10 @@ def test_spilled_registers_are_read_from_the_compiler_report(monkeypatch):
         "a.hip:90:1: remark: Function Name: _Zkernel_two [-Rpass-analysis=kernel-resource-usage]",
         "a.hip:90:1: remark:     SGPRs Spill: 0 [-Rpass-analysis=kernel-resource-usage]",
         "a.hip:90:1: remark:     VGPRs Spill: 0 [-Rpass-analysis=kernel-resource-usage]",
+        # accumulators kept in memory are reported as scratch, not as spills: 704 bytes a lane are 176 registers
+        "a.hip:95:1: remark: Function Name: _Zkernel_three [-Rpass-analysis=kernel-resource-usage]",
+        "a.hip:95:1: remark:     ScratchSize [bytes/lane]: 704 [-Rpass-analysis=kernel-resource-usage]",
+        "a.hip:95:1: remark:     VGPRs Spill: 0 [-Rpass-analysis=kernel-resource-usage]",
         "a.hip:5:3: warning: something else",
     ])
     logged = []
@@ -27,7 +31,7 @@ def test_spilled_registers_are_read_from_the_compiler_report(monkeypatch):
     monkeypatch.setattr(
         subprocess, "run", lambda *a, **k: subprocess.CompletedProcess(a, 0, stdout=report, stderr=None)
     )
-    assert build._run(["hipcc"], "compiling a.hip") == {"_Zkernel_one": 301, "_Zkernel_two": 0}
+    assert build._run(["hipcc"], "compiling a.hip") == {"_Zkernel_one": 301, "_Zkernel_two": 0, "_Zkernel_three": 176}
     assert any("warning: something else" in line and "remark" not in line for line in logged)
     assert not any("__global__" in line or "| ^" in line for line in logged)
     assert any("_Zkernel_one spills 301" in line for line in logged)
