@@ -277,6 +277,29 @@ def test_product_activations_and_multiplier(dtype, m, n, k):
         torch.testing.assert_close(got.double().cpu(), ref, **_tolerance(dtype))
 
 
+@pytest.mark.parametrize("dtype", GPU_CASES)
+@pytest.mark.parametrize("rows,size", [(1, 64), (7, 100), (300, 192), (3, 2048)])
+def test_norm_with_weights_stored_around_zero(dtype, rows, size):
+    from types import SimpleNamespace
+
+    from mini_llm_runtime_amd.parts import build_part
+    from mini_llm_runtime_amd.parts.spec import PartSpec
+
+    ops = _ops("hip", dtype)
+    g = torch.Generator().manual_seed(rows + size)
+    norm = build_part("norm", PartSpec("rms_norm", {"size": size, "eps": 1e-5, "weight_offset": 1.0}))
+    stored = (torch.randn(size, generator=g) * 0.3).to(torch.bfloat16)  # as a checkpoint holds it
+    norm.bind({"weight": stored.to(dtype).cuda()}, dtype=dtype, device=torch.device("cuda"))
+    assert norm.weight.dtype == torch.float32  # 1 + w does not fit bfloat16
+    x = torch.randn(rows, size, generator=g) * 3.0
+    delta = torch.randn(rows, size, generator=g).to(dtype)
+    stream = x.clone().cuda()
+    got = norm.forward(SimpleNamespace(ops=ops), stream, delta.cuda())
+    want = plain.zero_centred_rms_norm(x.double() + delta.double(), stored.double(), 1e-5)
+    torch.testing.assert_close(stream.cpu().double(), x.double() + delta.double(), rtol=1e-6, atol=1e-6)  # the 32-bit sum
+    torch.testing.assert_close(got.double().cpu(), want, **_tolerance(dtype))
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("experts,top,groups,keep", [(8, 2, 4, 2), (6, 1, 6, 3), (4, 4, 1, 1), (16, 3, 8, 3), (64, 6, 8, 4), (12, 3, 2, 1), (5, 2, 1, 1)])
 def test_routing_kernel(experts, top, groups, keep):
