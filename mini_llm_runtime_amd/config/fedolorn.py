@@ -77,7 +77,8 @@ class FedolornAttention:
 @dataclass(frozen=True)
 class FedolornFeedForward:
     """kind "dense": one feed-forward of `ff` inner features.  kind "moe": `experts` of them,
-    `top` per token, chosen among the best `groups_keep` of `groups_count` groups of neighbours."""
+    `top` per token; the experts are cut into `groups_count` contiguous blocks, and only those of the
+    `groups_keep` highest-scoring blocks are eligible."""
 
     kind: str
     ff: int

@@ -185,9 +185,9 @@ int mlr_sample_static(const float* logits, const float* temperature, const float
 
 // Routed experts (moe.hip).  mlr_moe_route: per token, from the router's float32 logits [tokens,
 // experts]: s = sigmoid(z), choice scores c = s + correction (float32 [experts], or null); the
-// experts form `groups` equal groups of neighbours, a group's score is the sum of its two largest
-// c, only experts of the `keep` best groups can be chosen; ids [tokens, top] are the `top` largest
-// c among those (ties to the lower index) and weights [tokens, top] their s times `scale`.
+// expert axis is cut into `groups` contiguous blocks of experts / groups; block score = top-2 sum of
+// c; eligible are the experts of the `keep` highest blocks; ids [tokens, top] = arg-top-`top` of c over
+// the eligible (ties to the lower index), weights [tokens, top] = s[id] * scale.
 int mlr_moe_route(const float* logits, const float* correction, int* ids, float* weights, int tokens, int experts,
                   int top, int groups, int keep, float scale, hipStream_t stream);
 // The (token, choice) pairs p = token * top + choice sorted by expert: sorted [pairs], offsets

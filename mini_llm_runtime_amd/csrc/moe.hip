@@ -29,9 +29,10 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
   }
 }
 
-// One wavefront per token.  s = sigmoid(z); choice score c = s + correction; a group's score is the
-// sum of its two largest c; experts outside the `keep` best groups get c = -inf; the `top` largest c
-// win, and a winner's weight is its s times `scale`.  Ties go to the lower index.
+// One wavefront per token.  s = sigmoid(z), c = s + correction; block g of experts / groups
+// consecutive experts scores top-2 sum of its c; c := -inf outside the `keep` highest blocks; then
+// `top` rounds of arg-max over c (ties to the lower index), each winner e leaving ids = e and
+// weights = s[e] * scale.
 __global__ __launch_bounds__(kWave) void moe_route_kernel(const float* __restrict__ logits,
                                                           const float* __restrict__ correction,
                                                           int* __restrict__ ids, float* __restrict__ weights,
@@ -52,7 +53,7 @@ __global__ __launch_bounds__(kWave) void moe_route_kernel(const float* __restric
   __syncthreads();
   if (groups > 1 && keep < groups) {
     for (int g = lane; g < groups; g += kWave) {
-      float a = -INFINITY, b = -INFINITY;  // the two largest of the group
+      float a = -INFINITY, b = -INFINITY;  // running top-2 of the block
       for (int e = g * per; e < (g + 1) * per; ++e) {
         const float v = c[e];
         if (v > a) {

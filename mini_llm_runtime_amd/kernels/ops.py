@@ -919,9 +919,10 @@ class HipOps:
         scale: float,
     ) -> tuple[torch.Tensor, torch.Tensor]:
         """Which experts every token uses (int32 [T, top]) and with what weight (float32 [T, top]),
-        from the router's float32 logits [T, experts]: sigmoid scores; the choice is made on score
-        + correction among the experts of the `keep_groups` best of `groups` groups of neighbours (a
-        group's score: the sum of its two largest); a chosen expert weighs its score times `scale`."""
+        from the router's float32 logits z [T, experts]: s = sigmoid(z), c = s + correction; the expert
+        axis is cut into `groups` contiguous blocks, a block scores the top-2 sum of its c, and ids are
+        the arg-top-`top` of c over the experts of the `keep_groups` highest blocks; weights = s[ids] *
+        `scale` (c only decides)."""
         self._check(logits, "router logits", torch.float32, (None, None))
         tokens, experts = logits.shape
         if correction is not None:

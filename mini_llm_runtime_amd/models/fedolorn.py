@@ -1,7 +1,7 @@
 """The Fedolorn decoder as a list of parts.
 
 A pre-norm decoder whose layers are listed one by one in its config.json, each with sizes of its
-own: RMSNorm with weights stored around zero; attention without any position encoding, with a
+own: RMSNorm whose checkpoint holds weight - 1; attention without any position encoding, with a
 mask cut into runs of positions, value heads of their own width, a scale from the config and a
 sigmoid output gate; then either a dense feed-forward with a squared ReLU, or a mixture of
 experts with sigmoid scores, a correction vector and a choice limited to the best groups, or

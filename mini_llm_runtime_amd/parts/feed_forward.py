@@ -84,12 +84,12 @@ class RoutedExperts(FeedForward):
     """A mixture of `experts` small feed-forwards (`down_e(act(up_e(x)))`, no biases) of which every
     token uses `top`.
 
-    Routing, all in 32-bit: z = Wr h; s = sigmoid(z); the choice is made on c = s + correction (a
-    stored vector that steers the load and takes no part in the weights).  The experts form
-    `groups` equal groups of neighbours; a group's score is the sum of its two largest c, only
-    experts of the `keep_groups` best groups can be chosen (for the others c counts as minus
-    infinity), and of those the `top` largest c win.  A chosen expert's output is weighted with
-    its s times `router_scale`; the weights are not renormalised.
+    Routing, all in 32-bit: z = Wr h, s = sigmoid(z), c = s + correction (a stored vector; c only
+    decides, the mixture's weights come from s).  The expert axis is cut into `groups` contiguous
+    blocks of experts / groups; block score = top-2 sum of its c; eligible = experts of the
+    `keep_groups` highest blocks (c := -inf elsewhere, since c may be negative); chosen = arg-top-`top`
+    of c over the eligible; y = sum over chosen e of (router_scale * s_e) * expert_e(h), with no
+    division by the sum of the weights.
 
     Everything runs on the device, so steps can be recorded: the routing kernel leaves expert ids
     and weights per token, an alignment kernel sorts the (token, choice) pairs by expert into row
