@@ -43,9 +43,9 @@ class GQAAttention(Mixer):
         (the larger, rounded up to a multiple of 16) with zero rows in the projections: zeros add
         nothing to a score, zero value dims come out as zeros and meet zero columns of the output
         projection.  The padding is made once, when the weights are bound.
-    output_gate: the merged heads are multiplied element by element with sigmoid(Wg h), h being
-        the mixer's own input, before the output projection.  The gate product runs behind the
-        attention kernel and multiplies in its epilogue.
+    output_gate: out = Wo (A * sigmoid(Wg h)), A the attended heads side by side [T, heads * value_dim],
+        * the Hadamard product, h the input that q, k and v are made from too.  The Wg product runs
+        behind the attention kernel and multiplies in its epilogue.
     """
 
     replayable = True
