@@ -92,3 +92,16 @@ class PendingScale:
     @property
     def shape(self) -> torch.Size:
         return self.h.shape
+
+
+@dataclass
+class NormedDelta:
+    """A part's output that enters the residual stream through a norm of its own:
+    x += weight * y * rsqrt(mean(y^2) + eps), for arrangements that norm a sublayer's output as well as
+    its input.  Handed to the next norm as its delta, so that the normed addition and that norm are one
+    kernel.  `y` is whatever a part may return: [T, H] in the engine's dtype or float32, a float32 stack
+    [S, T, H] whose sum it is, or a product that has not run."""
+
+    y: object
+    weight: torch.Tensor
+    eps: float

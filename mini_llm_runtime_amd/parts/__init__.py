@@ -1,6 +1,6 @@
 """Parts a layer is put together from, and the model that runs them."""
 
-from . import attention, block, feed_forward, norm, position  # noqa: F401  (register the built-in kinds)
+from . import attention, block, feed_forward, latent_attention, norm, position, retention, token_input  # noqa: F401  (register the built-in kinds)
 from .base import Block, FeedForward, Mixer, Norm, Part, PositionEncoding
 from .context import KVView, StateView, StepContext
 from .model import DecoderModel

@@ -7,6 +7,7 @@ from typing import Mapping, Optional
 import torch
 
 from .base import Block, FeedForward, Mixer, Norm, Part
+from ..kernels.pending import NormedDelta
 from .context import StepContext
 from .registry import register_part
 
@@ -54,6 +55,71 @@ class PreNormBlock(Block):
         h = _norm(self.norm_post_mixer, self.feed_forward, ctx, x, mixed)
         out = self.feed_forward.forward(ctx, h)
         return _stream_after(h, x), out
+
+
+@register_part("block", "sandwich_norm")
+class SandwichNormBlock(Block):
+    """Norms before AND after each sublayer:
+
+        x += norm_mixer_out(mixer(norm_input(x)));  x += norm_ff_out(feed_forward(norm_post_mixer(x)));
+        x += norm(token_input(x))      (if the layer has a token input; it reads the stream itself, un-normed)
+
+    A sublayer's output y enters the stream as w * y * rsqrt(mean(y^2) + eps), computed in 32-bit.  Each
+    such addition is one kernel with the norm (or the rounding of the stream to the engine's dtype)
+    that reads the stream next; the last one is handed to the next block as a `NormedDelta`.
+    A layer may have no feed-forward and no token input.
+    """
+
+    replayable = True
+
+    def __init__(
+        self,
+        mixer: Mixer,
+        feed_forward: Optional[FeedForward],
+        norms: Mapping[str, Norm],
+        token_input: Optional[Part] = None,
+    ) -> None:
+        needed = ["input", "mixer_out"] + (["post_mixer", "ff_out"] if feed_forward is not None else [])
+        missing = [n for n in needed if n not in norms]
+        if missing:
+            raise ValueError(f"sandwich_norm block needs the norms {needed}, missing {missing}")
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.token_input = token_input
+        self.norm_input = norms["input"]
+        self.norm_mixer_out = norms["mixer_out"]
+        self.norm_post_mixer = norms.get("post_mixer") if feed_forward is not None else None
+        self.norm_ff_out = norms.get("ff_out") if feed_forward is not None else None
+        for norm in (self.norm_mixer_out, self.norm_post_mixer, self.norm_ff_out):
+            if norm is not None and not hasattr(norm, "eps"):
+                raise ValueError("sandwich_norm takes RMS norms (a weight and an eps)")
+
+    def children(self) -> dict[str, Part]:
+        parts: dict[str, Part] = {"mixer": self.mixer, "norm_input": self.norm_input, "norm_mixer_out": self.norm_mixer_out}
+        if self.feed_forward is not None:
+            parts.update(feed_forward=self.feed_forward, norm_post_mixer=self.norm_post_mixer, norm_ff_out=self.norm_ff_out)
+        if self.token_input is not None:
+            parts["token_input"] = self.token_input
+        return parts
+
+    def forward(
+        self, ctx: StepContext, x: torch.Tensor, delta, site: int
+    ) -> tuple[torch.Tensor, Optional[NormedDelta]]:
+        ops = ctx.ops
+        h = self.norm_input.forward(ctx, x, delta)
+        mixed = self.mixer.forward(ctx, h, site)
+        owed = NormedDelta(mixed, self.norm_mixer_out.weight, self.norm_mixer_out.eps)
+        if self.feed_forward is not None:
+            h = ops.add_normed(
+                x, owed.y, owed.weight, owed.eps, next_weight=self.norm_post_mixer.weight, next_eps=self.norm_post_mixer.eps
+            )
+            out = self.feed_forward.forward(ctx, h)
+            owed = NormedDelta(out, self.norm_ff_out.weight, self.norm_ff_out.eps)
+        if self.token_input is not None:
+            stream = ops.add_normed(x, owed.y, owed.weight, owed.eps, cast=True)
+            fed = self.token_input.forward(ctx, stream)
+            owed = NormedDelta(fed, self.token_input.norm_weight, self.token_input.norm_eps)
+        return x, owed
 
 
 def _norm(norm: Norm, consumer: Part, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor]):

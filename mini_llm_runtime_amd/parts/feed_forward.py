@@ -45,6 +45,45 @@ class SwiGLU(FeedForward):
         return ops.linear(hidden, self.down_weight, None, for_stream=True)  # the next norm's delta
 
 
+@register_part("feed_forward", "clamped_glu")
+class ClampedGLU(FeedForward):
+    """Dense gated feed-forward with clamped halves and biases on all three products:
+
+        g = min(Wgate x + bgate, limit),  u = clamp(Wup x + bup, -limit, limit),
+        y = Wdown (g * sigmoid(alpha * g) * (u + 1)) + bdown.
+
+    Gate and up are one product over the rows [Wgate ; Wup]; the gating reads its 32-bit sums.
+    """
+
+    replayable = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, limit: float, alpha: float = 1.702) -> None:
+        if hidden_size <= 0 or intermediate_size <= 0 or not limit > 0:
+            raise ValueError("ClampedGLU sizes and limit must be > 0")
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        self.limit = float(limit)
+        self.alpha = float(alpha)
+        self.gate_up_weight: Optional[torch.Tensor] = None
+        self.gate_up_bias: Optional[torch.Tensor] = None
+        self.down_weight: Optional[torch.Tensor] = None
+        self.down_bias: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {
+            "gate_up_weight": ParamSpec((2 * self.intermediate_size, self.hidden_size)),
+            "gate_up_bias": ParamSpec((2 * self.intermediate_size,), keep_stored_precision=True),
+            "down_weight": ParamSpec((self.hidden_size, self.intermediate_size)),
+            "down_bias": ParamSpec((self.hidden_size,), keep_stored_precision=True),
+        }
+
+    def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
+        ops = ctx.ops
+        sums = ops.linear(h, self.gate_up_weight, self.gate_up_bias, out_dtype=torch.float32)
+        hidden = ops.glu_clamped(sums, self.limit, self.alpha)
+        return ops.linear(hidden, self.down_weight, self.down_bias, for_stream=True)
+
+
 ACTIVATIONS = ("relu2", "sigmoid")  # what `ops.linear(..., activation=)` applies to its sums
 
 

@@ -21,7 +21,10 @@ def _build_layer(spec: LayerSpec) -> Block:
     mixer = build_part("mixer", spec.mixer)
     feed_forward = build_part("feed_forward", spec.feed_forward) if spec.feed_forward is not None else None
     norms = {name: build_part("norm", s) for name, s in spec.norms.items()}
-    return build_part("block", PartSpec(spec.block), mixer=mixer, feed_forward=feed_forward, norms=norms)
+    extra = {}
+    if spec.token_input is not None:  # only arrangements that take one are handed one
+        extra["token_input"] = build_part("token_input", spec.token_input)
+    return build_part("block", PartSpec(spec.block), mixer=mixer, feed_forward=feed_forward, norms=norms, **extra)
 
 
 def _walk(prefix: str, part: Part) -> Iterator[tuple[str, Part]]:

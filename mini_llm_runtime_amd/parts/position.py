@@ -4,6 +4,8 @@ from __future__ import annotations
 
 from typing import Mapping, Optional
 
+import math
+
 import numpy as np
 import torch
 
@@ -22,12 +24,24 @@ class RotaryEmbedding(PositionEncoding):
     frequencies are computed once in float64 on the host; the angles and their
     cosines and sines are computed once per step for all layers that share this
     encoding's constants.
+
+    scaling: None, or the four numbers (factor, original, fast, slow) of a stretch for contexts
+    beyond the `original` length.  With dim(t) = r ln(original / (2 pi t)) / (2 ln theta), lo =
+    max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), r - 1) and ramp_j = clamp((j - lo) / max(hi -
+    lo, 0.001), 0, 1), pair j turns at f_j / factor * ramp_j + f_j * (1 - ramp_j): fast pairs keep
+    their frequency, slow ones are stretched by `factor`.  Cosines and sines are then multiplied by
+    0.1 ln(factor) + 1.
     """
 
     replayable = True
 
-
-    def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None) -> None:
+    def __init__(
+        self,
+        head_dim: int,
+        theta: float,
+        rotary_dim: Optional[int] = None,
+        scaling: Optional[Mapping[str, float]] = None,
+    ) -> None:
         rotary_dim = head_dim if rotary_dim is None else int(rotary_dim)
         if rotary_dim <= 0 or rotary_dim % 2 or rotary_dim > head_dim:
             raise ValueError("rotary_dim must be even and within head_dim")
@@ -38,15 +52,35 @@ class RotaryEmbedding(PositionEncoding):
         self.theta = float(theta)
         exponents = np.arange(0, rotary_dim, 2, dtype=np.float64) / rotary_dim
         self._inv_freq_host = 1.0 / (self.theta**exponents)
+        self.amplitude = 1.0
+        self.scaling = None
+        if scaling is not None:
+            factor, original = float(scaling["factor"]), float(scaling["original"])
+            fast, slow = float(scaling["fast"]), float(scaling["slow"])
+            if not (factor > 0 and original > 0 and fast > 0 and slow > 0):
+                raise ValueError("the numbers of a rotary scaling must be > 0")
+            self.scaling = (factor, original, fast, slow)
+
+            def pair_of(turns: float) -> float:  # the (fractional) pair that makes `turns` turns over `original` positions
+                return rotary_dim * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+
+            lo = max(math.floor(pair_of(fast)), 0)
+            hi = min(math.ceil(pair_of(slow)), rotary_dim - 1)
+            ramp = np.clip((np.arange(rotary_dim // 2, dtype=np.float64) - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+            self._inv_freq_host = self._inv_freq_host / factor * ramp + self._inv_freq_host * (1.0 - ramp)
+            self.amplitude = 0.1 * math.log(factor) + 1.0
         self.inv_freq: Optional[torch.Tensor] = None
 
     def bind(self, params: Mapping[str, torch.Tensor], *, dtype: torch.dtype, device: torch.device) -> None:
         self.inv_freq = torch.from_numpy(self._inv_freq_host).to(device)
 
     def rotation(self, ctx: StepContext):
-        key = ("rotary", self.rotary_dim, self.theta)
+        key = ("rotary", self.rotary_dim, self.theta, self.scaling)
         if key not in ctx.memo:
-            cos, sin = ctx.ops.rope_table(ctx.positions, self.inv_freq)
+            if self.amplitude != 1.0:
+                cos, sin = ctx.ops.rope_table(ctx.positions, self.inv_freq, amplitude=self.amplitude)
+            else:
+                cos, sin = ctx.ops.rope_table(ctx.positions, self.inv_freq)
             ctx.memo[key] = (cos, sin, self.rotary_dim)
         return ctx.memo[key]
 

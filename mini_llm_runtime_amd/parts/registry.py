@@ -9,7 +9,7 @@ from typing import Any, Callable
 
 from .spec import PartSpec
 
-CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block")
+CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "token_input")
 
 _REGISTRY: dict[str, dict[str, Callable[..., Any]]] = {c: {} for c in CATEGORIES}
 

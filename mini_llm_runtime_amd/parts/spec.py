@@ -37,12 +37,15 @@ class PartSpec:
 @dataclass(frozen=True)
 class LayerSpec:
     """One layer: an arrangement (`block`) of a mixer, a feed-forward (None: the layer has
-    none, if its arrangement allows that) and norms."""
+    none, if its arrangement allows that) and norms.  `token_input`: a part that feeds something
+    of the token itself into the stream at this layer (None: the layer has none); only
+    arrangements that know what to do with one take it."""
 
     block: str
     mixer: PartSpec
     feed_forward: Optional[PartSpec]
     norms: Mapping[str, PartSpec]
+    token_input: Optional[PartSpec] = None
 
 
 @dataclass(frozen=True)
@@ -66,9 +69,10 @@ class WeightRule:
     A rule may take only a part of the stored tensor, and several rules may read the same
     tensor (a checkpoint that stores q, k and v as one matrix, or all experts stacked):
     `source_index` picks [index] of the leading dimension, `transpose` swaps a matrix that is
-    stored [in, out], `source_rows` = (first, count) then takes rows of what is left, in that
-    order.  `source_shape` is the stored tensor's whole shape; it is needed whenever the part
-    taken is not the whole tensor."""
+    stored [in, out], `source_rows` = (first, count) then takes rows of what is left and
+    `source_cols` = (first, count) columns (of a matrix: a table that several layers share, each
+    with columns of its own), in that order.  `source_shape` is the stored tensor's whole shape;
+    it is needed whenever the part taken is not the whole tensor."""
 
     name: str
     dest: str
@@ -82,6 +86,7 @@ class WeightRule:
     source_index: Optional[int] = None
     source_rows: Optional[tuple[int, int]] = None
     transpose: bool = False
+    source_cols: Optional[tuple[int, int]] = None
 
     def part_shape(self, stored: tuple[int, ...]) -> tuple[int, ...]:
         """Shape of what this rule takes of a stored tensor of shape `stored`."""
@@ -99,6 +104,11 @@ class WeightRule:
             if not shape or first < 0 or count <= 0 or first + count > shape[0]:
                 raise ValueError(f"weight rule {self.name!r}: source_rows {self.source_rows} are outside {shape}")
             shape = (count, *shape[1:])
+        if self.source_cols is not None:
+            first, count = self.source_cols
+            if len(shape) != 2 or first < 0 or count <= 0 or first + count > shape[1]:
+                raise ValueError(f"weight rule {self.name!r}: source_cols {self.source_cols} are outside {shape}")
+            shape = (shape[0], count)
         return shape
 
     def take(self, tensor):
@@ -110,6 +120,9 @@ class WeightRule:
         if self.source_rows is not None:
             first, count = self.source_rows
             tensor = tensor[first : first + count]
+        if self.source_cols is not None:
+            first, count = self.source_cols
+            tensor = tensor[:, first : first + count]
         return tensor
 
     def dest_rows(self, count: int) -> "list[int]":

@@ -88,7 +88,7 @@ def _stored_shape(rule: WeightRule, p: ParamSpec) -> tuple[int, ...]:
     part = p.shape if rule.rows is None else (rule.rows, *p.shape[1:])
     if rule.source_shape is not None:
         stored = tuple(rule.source_shape)
-    elif rule.source_index is not None or rule.source_rows is not None:
+    elif rule.source_index is not None or rule.source_rows is not None or rule.source_cols is not None:
         raise ValueError(f"weight rule {rule.name!r} takes a part of its tensor and must give source_shape")
     else:
         stored = tuple(part[::-1]) if rule.transpose else tuple(part)

@@ -12,9 +12,12 @@ Each method has the signature and the contract of the method of the same name of
 
 from __future__ import annotations
 
+import math
 from typing import Optional
 
 import torch
+
+from mini_llm_runtime_amd.kernels.pending import NormedDelta
 
 
 class TorchOps:
@@ -27,13 +30,33 @@ class TorchOps:
         self.calls[name] = self.calls.get(name, 0) + 1
 
     # residual stream ------------------------------------------------------------------
-    def embedding(self, table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    def embedding(self, table: torch.Tensor, ids: torch.Tensor, out_dtype=None) -> torch.Tensor:
         self._count("embedding")
-        return table[ids.long()].float()
+        return table[ids.long()].to(out_dtype or torch.float32)
+
+    def settle(self, h):
+        if isinstance(h, NormedDelta):
+            y = self._sum(h.y)
+            return h.weight.float() * (y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + h.eps))
+        return h
+
+    @staticmethod
+    def _sum(y):
+        return y.float().sum(0) if y.dim() == 3 else y.float()
+
+    def add_normed(self, x, y, weight, eps, next_weight=None, next_eps=0.0, cast=False):
+        self._count("add_normed")
+        assert x.dtype == torch.float32
+        x += self.settle(NormedDelta(y, weight, eps))
+        if next_weight is not None:
+            return (next_weight.float() * (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + next_eps))).to(self.dtype)
+        return x.to(self.dtype) if cast else None
 
     def rmsnorm(self, x, weight, eps, delta=None):
         self._count("rmsnorm")
         assert x.dtype == torch.float32
+        if isinstance(delta, NormedDelta):
+            return self.add_normed(x, delta.y, delta.weight, delta.eps, next_weight=weight, next_eps=eps)
         if delta is not None:
             x += delta.float().sum(0) if delta.dim() == 3 else delta.float()
         variance = x.pow(2).mean(-1, keepdim=True)
@@ -48,6 +71,8 @@ class TorchOps:
             x.copy_(cap * torch.tanh(x / cap))
 
     def gather_rows(self, x, rows):
+        if isinstance(x, NormedDelta):
+            return NormedDelta(self.gather_rows(x.y, rows), x.weight, x.eps)
         return (x[:, rows.long()] if x.dim() == 3 else x[rows.long()]).contiguous()
 
     # matrix products ---------------------------------------------------------------------
@@ -63,6 +88,8 @@ class TorchOps:
             y = torch.clamp(y, min=0.0) ** 2
         elif activation == "sigmoid":
             y = torch.sigmoid(y)
+        elif activation == "gelu_tanh":
+            y = 0.5 * y * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (y + 0.044715 * y**3)))
         elif activation is not None:
             raise ValueError(activation)
         if multiply is not None:
@@ -80,9 +107,97 @@ class TorchOps:
         return (g * torch.sigmoid(g) * u).to(self.dtype)
 
     # positions and cache --------------------------------------------------------------------
-    def rope_table(self, positions, inv_freq):
+    def rope_table(self, positions, inv_freq, amplitude=1.0):
         ang = positions.double()[:, None] * inv_freq.double()[None, :]
-        return ang.cos().float(), ang.sin().float()
+        return (ang.cos() * amplitude).float(), (ang.sin() * amplitude).float()
+
+    def glu_clamped(self, sums, limit, alpha=1.702):
+        self._count("glu_clamped")
+        inter = sums.shape[1] // 2
+        g = sums[:, :inter].float().clamp(max=limit)
+        u = sums[:, inter:].float().clamp(-limit, limit)
+        return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(self.dtype)
+
+    @staticmethod
+    def _rotate(x, rotation):  # x [T, n, d] float32; the first r dims in two halves
+        if rotation is None:
+            return x
+        cos, sin, r = rotation
+        half = r // 2
+        a, b = x[..., :half], x[..., half:r]
+        c, s = cos[:, None, :], sin[:, None, :]
+        return torch.cat([a * c - b * s, b * c + a * s, x[..., r:]], dim=-1)
+
+    def latent_prepare(
+        self, projected, *, heads, head_dim, rot_dim, kv_rank, own_cache, gated, norm_weight, eps, rotation, slot_mapping,
+        key_pages, value_pages, block_size, kernel_dim,
+    ):
+        self._count("latent_prepare")
+        tokens = projected.shape[0]
+        p = projected.float()
+        q = p[:, : heads * (head_dim + rot_dim)].view(tokens, heads, head_dim + rot_dim)
+        at = heads * (head_dim + rot_dim)
+        q_plain = q[..., :head_dim].reshape(tokens, heads * head_dim).to(self.dtype)
+        q_latent = torch.zeros(tokens, heads, kernel_dim, dtype=torch.float32)
+        q_latent[..., kv_rank : kv_rank + rot_dim] = self._rotate(q[..., head_dim:], rotation)
+        if own_cache:
+            c = p[:, at : at + kv_rank]
+            c = norm_weight.float() * (c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps))
+            r = self._rotate(p[:, None, at + kv_rank : at + kv_rank + rot_dim], rotation)[:, 0]
+            at += kv_rank + rot_dim
+            row = torch.zeros(tokens, kernel_dim, dtype=torch.float32)
+            row[:, :kv_rank] = c
+            row[:, kv_rank : kv_rank + rot_dim] = r
+            value = torch.zeros(tokens, kernel_dim, dtype=torch.float32)
+            value[:, :kv_rank] = c
+            slots = slot_mapping.long()
+            ok = slots >= 0
+            page, off = slots[ok] // block_size, slots[ok] % block_size
+            key_pages[page, 0, off, :] = row[ok].to(key_pages.dtype)
+            value_pages[page, 0, :, off] = value[ok].to(value_pages.dtype)
+        gate = torch.sigmoid(p[:, at : at + heads]) if gated else None
+        return q_plain, q_latent.view(tokens, heads * kernel_dim).to(self.dtype), gate
+
+    def heads_linear(self, x, weight, *, in_stride, out=None, out_stride=None, row_scale=None):
+        self._count("heads_linear")
+        heads, n, k = weight.shape
+        tokens = x.shape[0]
+        xin = x.view(tokens, heads, in_stride)[..., :k].float()
+        y = torch.einsum("thk,hnk->thn", xin, weight.float())
+        if row_scale is not None:
+            y = y * row_scale.float()[..., None]
+        if out is None:
+            return y.reshape(tokens, heads * n).to(self.dtype)
+        out.view(tokens, heads, out_stride)[..., :n] = y.to(out.dtype)
+        return out
+
+    def retention_scan(
+        self, projected, state, read_rows, write_rows, ctx, *, heads, head_dim, value_dim, decay, key_scale, rotation
+    ):
+        self._count("retention_scan")
+        tokens = projected.shape[0]
+        p = projected.float()
+        qk = heads * head_dim
+        q = self._rotate(p[:, :qk].view(tokens, heads, head_dim), rotation)
+        k = self._rotate(p[:, qk : 2 * qk].view(tokens, heads, head_dim), rotation) * key_scale
+        v = p[:, 2 * qk : 2 * qk + heads * value_dim].view(tokens, heads, value_dim)
+        out = torch.zeros(tokens, heads, value_dim, dtype=torch.float32)
+        for r in range(ctx.num_entries):
+            a, b = int(ctx.cu_q[r]), int(ctx.cu_q[r + 1])
+            s = state[int(read_rows[r])].float().clone() if int(ctx.q_starts[r]) > 0 else torch.zeros_like(state[0])
+            for t in range(a, b):
+                s = decay.float()[:, None, None] * s + k[t][:, :, None] * v[t][:, None, :]
+                out[t] = torch.einsum("hdv,hd->hv", s, q[t])
+            state[int(write_rows[r])] = s
+        return out.view(tokens, heads * value_dim)
+
+    def retention_gate(self, retained, projected, *, heads, value_dim, gate_offset, eps):
+        self._count("retention_gate")
+        tokens = retained.shape[0]
+        o = retained.float().view(tokens, heads, value_dim)
+        o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+        z = projected[:, gate_offset : gate_offset + heads * value_dim].float()
+        return (o.reshape(tokens, heads * value_dim) * (z * torch.sigmoid(z))).to(self.dtype)
 
     def rope_kv_write(
         self, qkv, rotation, slot_mapping, key_pages, value_pages, *, num_heads, num_kv_heads, head_dim, block_size, write=True
@@ -119,7 +234,7 @@ class TorchOps:
 
     def paged_attention(
         self, qkv, key_pages, value_pages, block_table, ctx, *, num_heads, num_kv_heads, head_dim, block_size, scale, window,
-        defer_merge=False, plan=None, chunk=None,
+        defer_merge=False, plan=None, chunk=None, sinks=None,
     ):
         self._count("paged_attention")
         tokens = qkv.shape[0]
@@ -141,7 +256,12 @@ class TorchOps:
             k = k.repeat_interleave(group, dim=1)
             v = v.repeat_interleave(group, dim=1)
             s = torch.einsum("hd,nhd->hn", q[t], k) * scale
-            w = torch.softmax(s, dim=-1)
+            if sinks is not None:  # one more term of the denominator, with no key and no value
+                top = torch.maximum(s.max(-1).values, sinks.float())
+                e = torch.exp(s - top[:, None])
+                w = e / (e.sum(-1) + torch.exp(sinks.float() - top))[:, None]
+            else:
+                w = torch.softmax(s, dim=-1)
             out[t] = torch.einsum("hn,nhd->hd", w, v)
         return out.reshape(tokens, num_heads * head_dim).to(self.dtype)
 
