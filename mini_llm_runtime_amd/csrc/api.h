@@ -17,8 +17,9 @@ extern "C" {
 const char* mlr_last_error();
 int mlr_version();
 
-// out[t, :] = float(table[ids[t], :]); an id outside [0, vocab) gives a NaN row.
-int mlr_embedding(const void* table, int dtype, const int* ids, float* out, int tokens, int hidden,
+// out[t, :] = table[ids[t], :], as float32 (out_is_f32) or in the table's type; an id outside
+// [0, vocab) gives a NaN row.
+int mlr_embedding(const void* table, int dtype, const int* ids, void* out, int out_is_f32, int tokens, int hidden,
                   int vocab, hipStream_t stream);
 
 // x (float32 [rows, hidden]) += delta, then out = weight * x * rsqrt(mean(x^2) + eps)
@@ -43,9 +44,9 @@ int mlr_gather_rows(const void* src, const int* rows, void* out, int count, int6
 // out[m, i] = silu(gate_up[m, i]) * gate_up[m, inter + i].
 int mlr_silu_mul(const void* gate_up, void* out, int dtype, int rows, int inter, hipStream_t stream);
 
-// cos/sin [tokens, half] float32 of positions[t] * inv_freq[j], computed in float64.
+// cos/sin [tokens, half] float32 of positions[t] * inv_freq[j], times `amplitude`, computed in float64.
 int mlr_rope_table(const int* positions, const double* inv_freq, float* cos, float* sin, int tokens,
-                   int half, hipStream_t stream);
+                   int half, float amplitude, hipStream_t stream);
 
 // Rotate q and k of qkv [tokens, (heads + 2 kv_heads) * head_dim] in place (first
 // rotary_dim dims of every head, half-split pairs; rotary_dim 0: no rotation) and,
@@ -155,12 +156,47 @@ int mlr_gemm_merge_fused_bf16(const float* attn_partial, const int* context_lens
 // q is read from q[t * q_stride + head * head_dim + i]; out is [tokens, heads * head_dim];
 // pages are laid out as for mlr_rope_kv_write.
 // A page id outside [0, num_pages) among the visible keys gives a NaN row.
+// sinks (float32 [heads], or null): the softmax's denominator also holds exp(sinks[head]).
 int mlr_paged_attention_simple(const void* q, int64_t q_stride, const void* key_pages,
                                const void* value_pages, const int* block_table, int table_width,
                                const int* token_entry, const int* positions, void* out, int dtype,
                                int tokens, int entries, int heads, int kv_heads, int head_dim,
                                int block_size, int num_pages, float scale, int window, int chunk,
-                               hipStream_t stream);
+                               const float* sinks, hipStream_t stream);
+
+// x (float32 [rows, hidden], in place) += weight * y * rsqrt(mean(y^2) + eps), y [rows, hidden] float32
+// or `dtype`, or `slices` float32 partial sums [slices, rows, hidden].  Then mode 1: out = next_weight * x *
+// rsqrt(mean(x^2) + next_eps), mode 2: out = x, both in `dtype`; mode 0: no output.
+int mlr_add_normed(float* x, const void* y, int y_is_f32, int slices, const void* weight, int weight_is_f32, float eps,
+                   const void* next_weight, int next_is_f32, float next_eps, int mode, void* out, int dtype, int rows,
+                   int hidden, hipStream_t stream);
+
+// out[m, i] = g * sigmoid(alpha * g) * (u + 1), g = min(sums[m, i], limit), u = clamp(sums[m, inter + i],
+// -limit, limit).
+int mlr_glu_clamped(const void* sums, int sums_is_f32, void* out, int dtype, int rows, int inter, float limit,
+                    float alpha, hipStream_t stream);
+
+// What a latent-attention layer does between its input product and the attention kernels (see mixers.hip).
+int mlr_latent_prepare(const float* projected, int width, void* q_plain, void* q_latent, float* gate, const float* cos,
+                       const float* sin, int rotary_dims, const void* norm_weight, int weight_is_f32, float eps,
+                       const int* slots, void* key_pages, void* value_pages, int dtype, int tokens, int heads, int dim,
+                       int rot, int rank, int kernel_dim, int block_size, int num_pages, int own_cache, int gated,
+                       hipStream_t stream);
+
+// out[t * out_row + h * out_stride + j] = row_scale[t, h] * sum_i x[t * in_row + h * in_stride + i] * w[h, j, i].
+int mlr_heads_linear(const void* x, int64_t in_row, int in_stride, const void* w, void* out, int64_t out_row,
+                     int out_stride, const float* row_scale, int dtype, int tokens, int heads, int n, int k,
+                     hipStream_t stream);
+
+// Retention over every entry's tokens in order, from and to rows of the state banks (see mixers.hip).
+int mlr_retention_scan(const float* projected, int width, float* state, int state_rows, const int* read_rows,
+                       const int* write_rows, const int* cu_q, const int* q_starts, const float* decay,
+                       const float* cos, const float* sin, int rotary_dims, float key_scale, float* out, int entries,
+                       int heads, int dim, int vdim, hipStream_t stream);
+
+// out[t, h, :] = retained[t, h, :] / rms(retained[t, h, :]) * silu(projected[t, gate_offset + h * vdim + :]).
+int mlr_retention_gate(const float* retained, const float* projected, int width, int gate_offset, void* out, int dtype,
+                       int tokens, int heads, int vdim, float eps, hipStream_t stream);
 
 // tokens[k] = argmax(logits[k, :]) (first maximum), or, where temperature[k] > 0,
 // the first index whose cumulative exp((x - max) / temperature) exceeds

@@ -89,6 +89,18 @@ struct Softmax {
   float l;  // this lane's share of the sum (its own keys of every tile)
 };
 
+// A sink joins a finished softmax state: one more term exp(sink) of the denominator that has no key
+// and no value (a learned number per query head, not scaled).  `m` is the state's maximum in base 2;
+// returns the factor for the numerators and updates the denominator.
+__device__ __forceinline__ float join_sink(const float* __restrict__ sinks, int head, float m, float& den) {
+  if (sinks == nullptr) return 1.0f;
+  const float s2 = sinks[head] * 1.44269504088896340736f;
+  const float m_new = fmaxf(m, s2);
+  const float keep = (m == -INFINITY) ? 0.f : fast_exp2(m - m_new);
+  den = den * keep + fast_exp2(s2 - m_new);
+  return keep;
+}
+
 // ---- decode ---------------------------------------------------------------------------------
 constexpr int kDecodeWaves = D > 128 ? 2 : 4;  // bounded by the LDS the merge needs
 constexpr int kPartialStride = D + 2;  // numerator[D], max, denominator
@@ -164,7 +176,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out,
     float* __restrict__ partial, int heads, int kv_heads, int head_tiles, int block_size, int num_pages,
-    float scale, int window, int chunk, int part, int splits) {
+    float scale, int window, int chunk, int part, int splits, const float* __restrict__ sinks) {
   __shared__ float sm_acc[kDecodeWaves][16][D];
   __shared__ float sm_m[kDecodeWaves][16];
   __shared__ float sm_l[kDecodeWaves][16];
@@ -314,6 +326,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     }
     const int h = kvh * group + htile * 16 + c;
     if (splits == 1) {
+      num *= join_sink(sinks, h, mstar, den);  // with partitions the merge does this, once
       const float v = poisoned ? __builtin_nanf("") : num / den;
       out[(static_cast<int64_t>(t) * heads + h) * D + d] = f32_to_bf16(v);
     } else {
@@ -336,7 +349,8 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
                                                                   const int* __restrict__ cu_q,
                                                                   const int* __restrict__ context_lens,
                                                                   bf16* __restrict__ out, int heads, int window,
-                                                                  int chunk, int part, int all_splits) {
+                                                                  int chunk, int part, int all_splits,
+                                                                  const float* __restrict__ sinks) {
   const int entry = blockIdx.x;
   const int h = blockIdx.y;
   const int lane = threadIdx.x;
@@ -395,10 +409,11 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
     if (s0 >= splits) break;
     load_batch(s0);
   }
+  const float keep = join_sink(sinks, h, mstar, den);
 #pragma unroll
   for (int j = 0; j < (D + kWave - 1) / kWave; ++j) {
     const int d = lane + j * kWave;
-    if (d < D) out[(static_cast<int64_t>(t) * heads + h) * D + d] = f32_to_bf16(num[j] / den);
+    if (d < D) out[(static_cast<int64_t>(t) * heads + h) * D + d] = f32_to_bf16(num[j] * keep / den);
   }
 }
 
@@ -456,7 +471,7 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, const int* __restrict__ cu_q, const int* __restrict__ context_lens,
     bf16* __restrict__ out, int num_tiles, int heads, int kv_heads, int bs_shift, int num_pages, float scale,
-    int window, int chunk, float* __restrict__ partial) {
+    int window, int chunk, float* __restrict__ partial, const float* __restrict__ sinks) {
   // gridDim.y > 1: the keys of every tile are cut into that many runs, one workgroup each, which
   // leave their unnormalised results in `partial` for attn_prefill_merge (few tiles behind a long
   // context would otherwise be as many long chains on a few compute units).
@@ -828,7 +843,8 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
       continue;
     }
     if (q_ok[b]) {
-      const float inv = 1.0f / l;
+      const float keep = join_sink(sinks, head, m_run[b], l);
+      const float inv = keep / l;
       bf16* orow = out + (static_cast<int64_t>(t_first + qi[b]) * heads + head) * D;
 #pragma unroll
       for (int dt = 0; dt < kDimTiles; ++dt) {
@@ -849,7 +865,7 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
                                                                  const int* __restrict__ tiles,
                                                                  const int* __restrict__ cu_q,
                                                                  bf16* __restrict__ out, int heads, int splits,
-                                                                 int tile_q) {
+                                                                 int tile_q, const float* __restrict__ sinks) {
   const int tile = blockIdx.x / heads;
   const int head = blockIdx.x - tile * heads;
   const int entry = tiles[2 * tile];
@@ -873,9 +889,10 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
       num1 += w * row[d + 1];
       den += w * row[D + 1];
     }
+    const float keep = join_sink(sinks, head, mstar, den);
     bf16* orow = out + (static_cast<int64_t>(t_first + q0 + qq) * heads + head) * D;
-    orow[d] = f32_to_bf16(num0 / den);
-    orow[d + 1] = f32_to_bf16(num1 / den);
+    orow[d] = f32_to_bf16(num0 * keep / den);
+    orow[d + 1] = f32_to_bf16(num1 * keep / den);
   }
 }
 
@@ -905,7 +922,7 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
                          const int* block_table, int table_width, const int* cu_q, const int* context_lens,
                          void* out, float* partial, int entries, int heads, int kv_heads, int block_size,
                          int num_pages, float scale, int window, int chunk, int part, int splits, int merge,
-                         hipStream_t stream) {
+                         const float* sinks, hipStream_t stream) {
   MLR_REQUIRE(q && key_pages && value_pages && block_table && cu_q && context_lens && out, "null pointer");
   MLR_REQUIRE(entries > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "bad head counts");
   MLR_REQUIRE(block_size > 0 && block_size % 4 == 0, "block_size must be a multiple of 4");
@@ -931,7 +948,7 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
 #define MLR_DECODE(depth)                                                                                       \
   attn_decode_kernel<depth><<<grid, kDecodeWaves * kWave, 0, stream>>>(                                         \
       qp, q_stride, kp, vp, block_table, table_width, cu_q, context_lens, op, partial, heads, kv_heads,         \
-      head_tiles, block_size, num_pages, scale, window, chunk, part, splits)
+      head_tiles, block_size, num_pages, scale, window, chunk, part, splits, sinks)
   bool launched = false;
   if constexpr (kMaxDecodeDepth >= 4) {
     if (tiles_per_wave >= 4) {
@@ -948,9 +965,10 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
   if (!launched) MLR_DECODE(1);
 #undef MLR_DECODE
   MLR_LAUNCH_CHECK();
+  MLR_REQUIRE(sinks == nullptr || merge, "partitions left unmerged cannot carry sinks");
   if (splits > 1 && merge) {
     attn_decode_merge_kernel<<<dim3(entries, heads), kWave, 0, stream>>>(
-        partial, cu_q, context_lens, static_cast<bf16*>(out), heads, window, chunk, part, splits);
+        partial, cu_q, context_lens, static_cast<bf16*>(out), heads, window, chunk, part, splits, sinks);
     MLR_LAUNCH_CHECK();
   }
   return 0;
@@ -959,12 +977,13 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
 // The merge that mlr_attention_decode left out: out[t] of every single-token entry from its
 // partitions in `partial`.
 int mlr_attention_decode_merge(const float* partial, const int* cu_q, const int* context_lens, void* out, int entries,
-                               int heads, int window, int chunk, int part, int splits, hipStream_t stream) {
+                               int heads, int window, int chunk, int part, int splits, const float* sinks,
+                               hipStream_t stream) {
   MLR_REQUIRE(partial && cu_q && context_lens && out, "null pointer");
   MLR_REQUIRE(entries > 0 && heads > 0 && heads <= 65535, "bad sizes");
   MLR_REQUIRE(part > 0 && part % 64 == 0 && splits > 1 && window >= 0 && chunk >= 0, "bad partitions");
   attn_decode_merge_kernel<<<dim3(entries, heads), kWave, 0, stream>>>(partial, cu_q, context_lens,
-                                                                      static_cast<bf16*>(out), heads, window, chunk, part, splits);
+                                                                      static_cast<bf16*>(out), heads, window, chunk, part, splits, sinks);
   MLR_LAUNCH_CHECK();
   return 0;
 }
@@ -989,7 +1008,7 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
                           const int* block_table, int table_width, const int* tiles, int num_tiles, int wide,
                           const int* cu_q, const int* context_lens, void* out, int heads, int kv_heads,
                           int block_size, int num_pages, float scale, int window, int chunk, int splits,
-                          float* partial, hipStream_t stream) {
+                          float* partial, const float* sinks, hipStream_t stream) {
   MLR_REQUIRE(splits >= 1 && splits <= 64, "splits must lie within 1..64");
   MLR_REQUIRE(splits == 1 || partial != nullptr, "several key runs need scratch memory");
   MLR_REQUIRE(q && key_pages && value_pages && block_table && tiles && cu_q && context_lens && out, "null pointer");
@@ -1033,12 +1052,14 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
       attn_prefill_kernel<qb, true><<<grid, 256 * kKeyGroups, kPrefillLds, stream>>>(                         \
           static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),                         \
           static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,         \
-          static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window, chunk, partial);  \
+          static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window, chunk, partial,  \
+          splits > 1 ? nullptr : sinks);  \
     else                                                                                                      \
       attn_prefill_kernel<qb, false><<<grid, 256 * kKeyGroups, kPrefillLds, stream>>>(                        \
           static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),                         \
           static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,         \
-          static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window, chunk, partial);  \
+          static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window, chunk, partial,  \
+          splits > 1 ? nullptr : sinks);  \
   } while (0)
   if constexpr (D <= 128) {
     if (wide)
@@ -1053,7 +1074,7 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
   if (splits > 1) {
     const int tile_q = (wide && D <= 128) ? 2 * kTileQ : kTileQ;
     attn_prefill_merge_kernel<<<dim3(static_cast<unsigned>(num_tiles) * heads), 256, 0, stream>>>(
-        partial, tiles, cu_q, static_cast<bf16*>(out), heads, splits, tile_q);
+        partial, tiles, cu_q, static_cast<bf16*>(out), heads, splits, tile_q, sinks);
     MLR_LAUNCH_CHECK();
   }
   return 0;

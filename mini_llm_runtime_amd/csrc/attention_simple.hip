@@ -21,7 +21,8 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ key_pages,
     const T* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ token_entry, const int* __restrict__ positions, T* __restrict__ out, int entries,
-    int heads, int kv_heads, int head_dim, int block_size, int num_pages, float scale, int window, int chunk) {
+    int heads, int kv_heads, int head_dim, int block_size, int num_pages, float scale, int window, int chunk,
+    const float* __restrict__ sinks) {
   __shared__ float qs[kMaxHeadDim];
   __shared__ float ps[kWave];
   __shared__ int64_t offs[kWave];
@@ -96,6 +97,15 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     __syncthreads();
   }
 
+  // a sink: one more term exp(sink) of the denominator, with no key and no value
+  if (sinks != nullptr) {
+    const float sink = sinks[h];
+    const float m_new = fmaxf(m, sink);
+    const float alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
+    l = l * alpha + expf(sink - m_new);
+#pragma unroll
+    for (int j = 0; j < kMaxHeadDim / kWave; ++j) acc[j] *= alpha;
+  }
   const bool any_bad = __any(bad);
   const float inv = 1.0f / l;
 #pragma unroll
@@ -114,7 +124,7 @@ extern "C" int mlr_paged_attention_simple(const void* q, int64_t q_stride, const
                                           const int* token_entry, const int* positions, void* out, int dtype,
                                           int tokens, int entries, int heads, int kv_heads, int head_dim,
                                           int block_size, int num_pages, float scale, int window, int chunk,
-                                          hipStream_t stream) {
+                                          const float* sinks, hipStream_t stream) {
   MLR_REQUIRE(q && key_pages && value_pages && block_table && token_entry && positions && out, "null pointer");
   MLR_REQUIRE(tokens > 0 && entries > 0 && heads > 0 && kv_heads > 0, "sizes must be > 0");
   MLR_REQUIRE(heads % kv_heads == 0, "query heads must be a multiple of KV heads");
@@ -130,12 +140,14 @@ extern "C" int mlr_paged_attention_simple(const void* q, int64_t q_stride, const
     paged_attention_simple_kernel<float><<<grid, kWave, 0, stream>>>(
         static_cast<const float*>(q), q_stride, static_cast<const float*>(key_pages),
         static_cast<const float*>(value_pages), block_table, table_width, token_entry, positions,
-        static_cast<float*>(out), entries, heads, kv_heads, head_dim, block_size, num_pages, scale, window, chunk);
+        static_cast<float*>(out), entries, heads, kv_heads, head_dim, block_size, num_pages, scale, window, chunk,
+        sinks);
   else
     paged_attention_simple_kernel<bf16><<<grid, kWave, 0, stream>>>(
         static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),
         static_cast<const bf16*>(value_pages), block_table, table_width, token_entry, positions,
-        static_cast<bf16*>(out), entries, heads, kv_heads, head_dim, block_size, num_pages, scale, window, chunk);
+        static_cast<bf16*>(out), entries, heads, kv_heads, head_dim, block_size, num_pages, scale, window, chunk,
+        sinks);
   MLR_LAUNCH_CHECK();
   return 0;
 }

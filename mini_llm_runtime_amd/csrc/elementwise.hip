@@ -13,19 +13,19 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // ---- embedding -------------------------------------------------------------------
 // qwen_model_runner.py:263 (F.embedding): a row gather, no scaling.
-template <typename T>
+template <typename T, typename TO>
 __global__ __launch_bounds__(256) void embedding_kernel(const T* __restrict__ table,
                                                         const int* __restrict__ ids,
-                                                        float* __restrict__ out, int hidden, int vocab) {
+                                                        TO* __restrict__ out, int hidden, int vocab) {
   const int t = blockIdx.x;
   const int id = ids[t];
-  float* dst = out + static_cast<int64_t>(t) * hidden;
+  TO* dst = out + static_cast<int64_t>(t) * hidden;
   if (id < 0 || id >= vocab) {
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = __builtin_nanf("");
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = from_f32<TO>(__builtin_nanf(""));
     return;
   }
   const T* src = table + static_cast<int64_t>(id) * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32(src[i]);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = from_f32<TO>(to_f32(src[i]));
 }
 
 // ---- RMSNorm (+ residual addition) ---------------------------------------------------
@@ -197,14 +197,15 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ gat
 __global__ __launch_bounds__(256) void rope_table_kernel(const int* __restrict__ positions,
                                                          const double* __restrict__ inv_freq,
                                                          float* __restrict__ cos_out,
-                                                         float* __restrict__ sin_out, int tokens, int half) {
+                                                         float* __restrict__ sin_out, int tokens, int half,
+                                                         double amplitude) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= static_cast<int64_t>(tokens) * half) return;
   const int t = static_cast<int>(i / half);
   const int j = static_cast<int>(i - static_cast<int64_t>(t) * half);
   const double angle = static_cast<double>(positions[t]) * inv_freq[j];
-  cos_out[i] = static_cast<float>(cos(angle));
-  sin_out[i] = static_cast<float>(sin(angle));
+  cos_out[i] = static_cast<float>(cos(angle) * amplitude);
+  sin_out[i] = static_cast<float>(sin(angle) * amplitude);
 }
 
 // ---- rotary encoding + paged key/value store ------------------------------------------
@@ -420,15 +421,20 @@ extern "C" {
 
 int mlr_version() { return 1; }
 
-int mlr_embedding(const void* table, int dtype, const int* ids, float* out, int tokens, int hidden,
+int mlr_embedding(const void* table, int dtype, const int* ids, void* out, int out_is_f32, int tokens, int hidden,
                   int vocab, hipStream_t stream) {
   MLR_REQUIRE(table && ids && out, "null pointer");
   MLR_REQUIRE(tokens > 0 && hidden > 0 && vocab > 0, "sizes must be > 0");
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
   if (dtype == kF32)
-    embedding_kernel<float><<<tokens, 256, 0, stream>>>(static_cast<const float*>(table), ids, out, hidden, vocab);
+    embedding_kernel<float, float><<<tokens, 256, 0, stream>>>(static_cast<const float*>(table), ids,
+                                                               static_cast<float*>(out), hidden, vocab);
+  else if (out_is_f32)
+    embedding_kernel<bf16, float><<<tokens, 256, 0, stream>>>(static_cast<const bf16*>(table), ids,
+                                                              static_cast<float*>(out), hidden, vocab);
   else
-    embedding_kernel<bf16><<<tokens, 256, 0, stream>>>(static_cast<const bf16*>(table), ids, out, hidden, vocab);
+    embedding_kernel<bf16, bf16><<<tokens, 256, 0, stream>>>(static_cast<const bf16*>(table), ids,
+                                                             static_cast<bf16*>(out), hidden, vocab);
   MLR_LAUNCH_CHECK();
   return 0;
 }
@@ -514,13 +520,14 @@ int mlr_silu_mul(const void* gate_up, void* out, int dtype, int rows, int inter,
 }
 
 int mlr_rope_table(const int* positions, const double* inv_freq, float* cos, float* sin, int tokens, int half,
-                   hipStream_t stream) {
+                   float amplitude, hipStream_t stream) {
   MLR_REQUIRE(positions && inv_freq && cos && sin, "null pointer");
   MLR_REQUIRE(tokens > 0 && half > 0, "sizes must be > 0");
   const int64_t total = static_cast<int64_t>(tokens) * half;
   const int64_t blocks = (total + 255) / 256;
   MLR_REQUIRE(blocks < (1ll << 31), "too many elements");
-  rope_table_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(positions, inv_freq, cos, sin, tokens, half);
+  rope_table_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(positions, inv_freq, cos, sin, tokens, half,
+                                                                       static_cast<double>(amplitude));
   MLR_LAUNCH_CHECK();
   return 0;
 }

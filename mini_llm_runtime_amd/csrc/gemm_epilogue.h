@@ -33,6 +33,7 @@ constexpr int kEpNone = 0;
 constexpr int kEpSwiglu = 1;
 constexpr int kEpRelu2 = 2;
 constexpr int kEpSigmoid = 3;
+constexpr int kEpGeluTanh = 4;  // 0.5 v (1 + tanh(sqrt(2 / pi) (v + 0.044715 v^3)))
 
 // The scaling factors of rows m0 .. m0 + count - 1 into `scales` (LDS), by all wavefronts of the
 // workgroup (a whole number of them): wavefront w takes the rows w, w + waves, ..., its lanes the
@@ -148,6 +149,13 @@ __device__ __forceinline__ void store4(const GemmEpilogue& ep, int64_t m, int n,
     } else if (ep.swiglu == kEpSigmoid) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] = 1.0f / (1.0f + __expf(-v[i]));
+    } else if (ep.swiglu == kEpGeluTanh) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        // 0.5 (1 + tanh(u)) = 1 / (1 + exp(-2 u))
+        const float u = 0.7978845608028654f * (v[i] + 0.044715f * v[i] * v[i] * v[i]);
+        v[i] = v[i] / (1.0f + __expf(-2.0f * u));
+      }
     }
     if (ep.multiply != nullptr) {
       const bf16* other = static_cast<const bf16*>(ep.multiply) + at;

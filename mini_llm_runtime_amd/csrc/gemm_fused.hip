@@ -458,7 +458,7 @@ int mlr_gemm_norm_fused_bf16(const float* x_in, float* x_out, const void* delta,
   }
   MLR_REQUIRE(w && y && n > 0, "null pointer or empty product");
   MLR_REQUIRE(reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0, "w and y must be 16-byte aligned");
-  MLR_REQUIRE(swiglu >= kEpNone && swiglu <= kEpSigmoid, "unknown epilogue");
+  MLR_REQUIRE(swiglu >= kEpNone && swiglu <= kEpGeluTanh, "unknown epilogue");
   MLR_REQUIRE(swiglu != kEpSwiglu || (n % 4 == 0 && bias == nullptr), "swiglu needs n % 4 == 0 and no bias");
   MLR_REQUIRE(row_blocks == 0 || row_blocks == 1 || row_blocks == 2, "row_blocks must be 0 (chosen), 1 or 2");
   const GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu};

@@ -1136,7 +1136,7 @@ int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f3
                   int swiglu, int slices, int kernel, int m, int n, int k, const float* row_sumsq, int sumsq_parts,
                   float norm_eps, const void* multiply, hipStream_t stream) {
   MLR_REQUIRE(x && w && y, "null pointer");
-  MLR_REQUIRE(swiglu >= kEpNone && swiglu <= kEpSigmoid, "unknown epilogue");
+  MLR_REQUIRE(swiglu >= kEpNone && swiglu <= kEpGeluTanh, "unknown epilogue");
   MLR_REQUIRE(multiply == nullptr || (swiglu != kEpSwiglu && slices == 1), "a multiplier goes with whole, unpaired sums");
   MLR_REQUIRE(slices == 1 || swiglu == kEpNone, "partial sums take no activation");
   MLR_REQUIRE(m > 0 && n > 0 && k > 0, "sizes must be > 0");

@@ -94,6 +94,8 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
         v *= v;
       } else if (swiglu == 3) {
         v = 1.0f / (1.0f + expf(-v));
+      } else if (swiglu == 4) {
+        v = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
       }
       if (multiply != nullptr) v *= to_f32(multiply[gm * N + gn]);
       if (out_is_f32)
@@ -116,7 +118,7 @@ extern "C" int mlr_gemm_simple(const void* x, const void* w, const void* bias, i
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
   MLR_REQUIRE(dtype == kBF16 || (out_is_f32 && (bias == nullptr || bias_is_f32)),
               "a float32 product has float32 bias and output");
-  MLR_REQUIRE(swiglu >= 0 && swiglu <= 3, "unknown epilogue");
+  MLR_REQUIRE(swiglu >= 0 && swiglu <= 4, "unknown epilogue");
   MLR_REQUIRE(swiglu != 1 || (n % 4 == 0 && bias == nullptr && multiply == nullptr),
               "swiglu needs n % 4 == 0, no bias and no multiplier");
   dim3 grid((n + kTN - 1) / kTN, (m + kTM - 1) / kTM);

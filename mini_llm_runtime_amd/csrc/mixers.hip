@@ -1,0 +1,472 @@
+// Kernels of mixers and arrangements beyond grouped-query attention: a sublayer's output added
+// to the stream through a norm of its own, the gating of a clamped feed-forward, what a
+// latent-attention layer does between its input product and the attention kernels, products with
+// one small matrix per head, and retention (linear attention with a decaying matrix state).
+// All arithmetic is float32; bfloat16 only exists in memory.
+#include "api.h"
+#include "common.h"
+
+namespace mlr {
+
+// ---- x += weight * y * rsqrt(mean(y^2) + eps), then what reads the stream next -----------------
+// y is one tensor (float32 or the engine's dtype) or `slices` float32 partial sums added in slice
+// order.  mode 1: out = next_weight * x * rsqrt(mean(x^2) + next_eps); mode 2: out = x rounded to the
+// engine's dtype; mode 0: nothing more.  One workgroup per row; the row stays in LDS between the
+// passes, and a thread only ever reads the elements it wrote itself.
+template <typename T>
+__global__ __launch_bounds__(256) void add_normed_kernel(float* __restrict__ x, const void* __restrict__ y,
+                                                         int y_is_f32, int slices, int rows,
+                                                         const void* __restrict__ weight, int weight_is_f32, float eps,
+                                                         const void* __restrict__ next_weight, int next_is_f32,
+                                                         float next_eps, int mode, T* __restrict__ out, int hidden) {
+  extern __shared__ float row_lds[];
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += 256) {
+    float v;
+    if (slices > 0) {
+      v = 0.f;
+      const float* p = static_cast<const float*>(y);
+      for (int s = 0; s < slices; ++s) v += p[(static_cast<int64_t>(s) * rows + row) * hidden + i];
+    } else {
+      v = y_is_f32 ? static_cast<const float*>(y)[row * hidden + i] : to_f32(static_cast<const T*>(y)[row * hidden + i]);
+    }
+    row_lds[i] = v;
+    ss += v * v;
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(hidden) + eps);
+  float* xr = x + row * hidden;
+  float ss2 = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += 256) {
+    const float v = xr[i] + (row_lds[i] * inv) * load_as_f32(weight, i, weight_is_f32);
+    xr[i] = v;
+    row_lds[i] = v;
+    ss2 += v * v;
+  }
+  if (mode == 0) return;
+  T* orow = out + row * hidden;
+  if (mode == 2) {
+    for (int i = threadIdx.x; i < hidden; i += 256) orow[i] = from_f32<T>(row_lds[i]);
+    return;
+  }
+  const float inv2 = 1.0f / sqrtf(block_sum(ss2, scratch) / static_cast<float>(hidden) + next_eps);
+  for (int i = threadIdx.x; i < hidden; i += 256)
+    orow[i] = from_f32<T>(load_as_f32(next_weight, i, next_is_f32) * (row_lds[i] * inv2));
+}
+
+// ---- g = min(gate, limit), u = clamp(up, -limit, limit): g * sigmoid(alpha g) * (u + 1) ---------
+// sums [rows, 2 * inter]: the gate sums, then the up sums.
+template <typename TI, typename T>
+__global__ __launch_bounds__(256) void glu_clamped_kernel(const TI* __restrict__ sums, T* __restrict__ out, int rows,
+                                                          int inter, float limit, float alpha) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= static_cast<int64_t>(rows) * inter) return;
+  const int64_t m = i / inter;
+  const int64_t c = i - m * inter;
+  const float g = fminf(to_f32(sums[m * 2 * inter + c]), limit);
+  const float u = fminf(fmaxf(to_f32(sums[m * 2 * inter + inter + c]), -limit), limit);
+  out[i] = from_f32<T>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+}
+
+// ---- latent attention: between the input product and the attention kernels ----------------------
+// `p` [tokens, width] float32 holds, per token: the queries (per head `dim` unrotated then `rot`
+// rotated dims), then (own_cache) the latent of `rank` dims and the shared key part of `rot` dims,
+// then (gated) one gate logit per head.  Per token this
+//  * rounds the unrotated query parts into q_plain [tokens, heads * dim],
+//  * rotates the rotated query parts into columns rank .. rank + rot of every head's latent query
+//    (q_latent [tokens, heads * D]; columns beyond rank + rot are cleared, the first `rank` belong
+//    to the product that follows),
+//  * (own_cache) norms the latent (weight, eps), rotates the key part, and stores the row
+//    [latent ; key part ; 0] at slot[t] of the key pages [page, 1, offset, D] and [latent ; 0]
+//    of the value pages [page, 1, D, offset]; a negative slot stores nothing,
+//  * (gated) gate[t, head] = sigmoid(logit), float32.
+// The rotation takes the first `rdims` of the `rot` dims in two halves (pair j, j + rdims / 2).
+template <typename T>
+__global__ __launch_bounds__(256) void latent_prepare_kernel(
+    const float* __restrict__ p, int width, T* __restrict__ q_plain, T* __restrict__ q_latent,
+    float* __restrict__ gate, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rdims,
+    const void* __restrict__ norm_weight, int weight_is_f32, float eps, const int* __restrict__ slots,
+    T* __restrict__ key_pages, T* __restrict__ value_pages, int heads, int dim, int rot, int rank, int D,
+    int block_size, int num_pages, int own_cache, int gated) {
+  __shared__ float scratch[16];
+  const int64_t t = blockIdx.x;
+  const float* row = p + t * width;
+  const int half = rdims / 2;
+  const float* cs = cos_t ? cos_t + t * half : nullptr;
+  const float* sn = sin_t ? sin_t + t * half : nullptr;
+  auto rotated = [&](const float* part, int j) {  // dim j of a rotated part of `rot` dims
+    if (j >= rdims || cs == nullptr) return part[j];
+    return j < half ? part[j] * cs[j] - part[j + half] * sn[j] : part[j] * cs[j - half] + part[j - half] * sn[j - half];
+  };
+  const int qd = dim + rot;
+  for (int i = threadIdx.x; i < heads * dim; i += 256) {
+    const int h = i / dim;
+    q_plain[t * heads * dim + i] = from_f32<T>(row[h * qd + (i - h * dim)]);
+  }
+  const int tail = D - rank;  // columns of a latent query that this kernel owns
+  for (int i = threadIdx.x; i < heads * tail; i += 256) {
+    const int h = i / tail;
+    const int j = i - h * tail;
+    q_latent[(t * heads + h) * D + rank + j] = from_f32<T>(j < rot ? rotated(row + h * qd + dim, j) : 0.f);
+  }
+  int at = heads * qd;
+  if (own_cache) {
+    const float* c = row + at;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < rank; i += 256) ss += c[i] * c[i];
+    const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(rank) + eps);
+    const int slot = slots[t];
+    if (slot >= 0) {
+      const int page = slot / block_size;
+      const int off = slot - page * block_size;
+      if (page < num_pages) {
+        T* krow = key_pages + (static_cast<int64_t>(page) * block_size + off) * D;
+        T* vcol = value_pages + static_cast<int64_t>(page) * D * block_size + off;
+        for (int i = threadIdx.x; i < D; i += 256) {
+          float kv = 0.f, vv = 0.f;
+          if (i < rank) {
+            kv = vv = (c[i] * inv) * load_as_f32(norm_weight, i, weight_is_f32);
+          } else if (i < rank + rot) {
+            kv = rotated(c + rank, i - rank);
+          }
+          krow[i] = from_f32<T>(kv);
+          vcol[static_cast<int64_t>(i) * block_size] = from_f32<T>(vv);
+        }
+      }
+    }
+    at += rank + rot;
+  }
+  if (gated)
+    for (int h = threadIdx.x; h < heads; h += 256) gate[t * heads + h] = 1.0f / (1.0f + expf(-row[at + h]));
+}
+
+// ---- one small matrix per head --------------------------------------------------------------------
+// y[t, h, n] = sum_k x[t, h * in_stride + k] * w[h, n, k]  (times row_scale[t, h], float32, if given),
+// stored at out[t * out_row + h * out_stride + n].  Plain float32 arithmetic, 64 x 64 output tile per
+// workgroup and head, 16-wide slices of k through LDS, 4 x 4 outputs a lane.
+template <typename T>
+__global__ __launch_bounds__(256) void heads_linear_kernel(const T* __restrict__ x, int64_t in_row, int in_stride,
+                                                           const T* __restrict__ w, T* __restrict__ out,
+                                                           int64_t out_row, int out_stride,
+                                                           const float* __restrict__ row_scale, int heads, int M,
+                                                           int N, int K) {
+  __shared__ float xs[16][64 + 4];
+  __shared__ float ws[16][64 + 4];
+  const int tid = threadIdx.x;
+  const int tm = tid / 16;
+  const int tn = tid % 16;
+  const int h = blockIdx.z;
+  const int64_t m0 = static_cast<int64_t>(blockIdx.y) * 64;
+  const int64_t n0 = static_cast<int64_t>(blockIdx.x) * 64;
+  const T* xh = x + static_cast<int64_t>(h) * in_stride;
+  const T* wh = w + static_cast<int64_t>(h) * N * K;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += 16) {
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int idx = tid + it * 256;
+      const int r = idx / 16;
+      const int kk = idx % 16;
+      const int64_t gk = k0 + kk;
+      xs[kk][r] = (m0 + r < M && gk < K) ? to_f32(xh[(m0 + r) * in_row + gk]) : 0.f;
+      ws[kk][r] = (n0 + r < N && gk < K) ? to_f32(wh[(n0 + r) * K + gk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = xs[kk][tm * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = ws[kk][tn * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t gm = m0 + tm * 4 + i;
+    if (gm >= M) continue;
+    const float s = row_scale ? row_scale[gm * heads + h] : 1.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t gn = n0 + tn * 4 + j;
+      if (gn < N) out[gm * out_row + static_cast<int64_t>(h) * out_stride + gn] = from_f32<T>(acc[i][j] * s);
+    }
+  }
+}
+
+// ---- retention ------------------------------------------------------------------------------------
+// S_t = decay S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per (entry, head), the entry's tokens in order.
+// `p` [tokens, width] float32 holds q (heads * dim), k (heads * dim), v (heads * vdim) and more; q and
+// k are rotated here (first rdims dims of a head in two halves) and k scaled by key_scale, all in
+// float32.  A wavefront owns 16 columns of one head's state: lane = (group of dims g = lane / 16,
+// column c = lane % 16) keeps S[d][c] for d = 4 i + g in registers.  Tokens are taken kBatch at a
+// time: their rotated q and k and their v go to LDS first, so the trip to memory is paid once per
+// batch and the chain from token to token is arithmetic only.  The state is read from row
+// read_rows[entry] of `state` [rows, heads, dim, vdim] (zeros when the entry starts its request) and
+// left in row write_rows[entry].  out [tokens, heads * vdim] float32.
+constexpr int kRetBatch = 8;
+
+template <int DPL>  // dims per lane: dim <= 4 * DPL
+__global__ __launch_bounds__(64) void retention_scan_kernel(
+    const float* __restrict__ p, int width, float* __restrict__ state, const int* __restrict__ read_rows,
+    const int* __restrict__ write_rows, const int* __restrict__ cu_q, const int* __restrict__ q_starts,
+    const float* __restrict__ decay, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rdims,
+    float key_scale, float* __restrict__ out, int heads, int dim, int vdim) {
+  __shared__ float qs[kRetBatch][4 * DPL];
+  __shared__ float ks[kRetBatch][4 * DPL];
+  __shared__ float vs[kRetBatch][16];
+  const int entry = blockIdx.x;
+  const int h = blockIdx.y;
+  const int v0 = blockIdx.z * 16;
+  const int lane = threadIdx.x;
+  const int g = lane / 16;
+  const int c = lane % 16;
+  const bool column = v0 + c < vdim;
+  const int t_first = cu_q[entry];
+  const int t_end = cu_q[entry + 1];
+  const float gamma = decay[h];
+  const int half = rdims / 2;
+  const int64_t head_state = static_cast<int64_t>(dim) * vdim;
+
+  float S[DPL];
+  const bool carried = q_starts[entry] > 0;
+  const float* src = state + (static_cast<int64_t>(read_rows[entry]) * heads + h) * head_state;
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) {
+    const int d = 4 * i + g;
+    S[i] = (carried && column && d < dim) ? src[static_cast<int64_t>(d) * vdim + v0 + c] : 0.f;
+  }
+
+  for (int tb = t_first; tb < t_end; tb += kRetBatch) {
+    const int count = min(kRetBatch, t_end - tb);
+    __syncthreads();  // the batch before is done with
+    for (int idx = lane; idx < count * dim; idx += 64) {
+      const int u = idx / dim;
+      const int d = idx - u * dim;
+      const int64_t t = tb + u;
+      const float* q = p + t * width + static_cast<int64_t>(h) * dim;
+      const float* k = q + static_cast<int64_t>(heads) * dim;
+      float qv = q[d], kv = k[d];
+      if (d < rdims && cos_t != nullptr) {
+        const int j = d < half ? d : d - half;
+        const float cv = cos_t[t * half + j], sv = sin_t[t * half + j];
+        const int partner = d < half ? d + half : d - half;
+        const float sign = d < half ? -1.f : 1.f;
+        qv = qv * cv + sign * q[partner] * sv;
+        kv = kv * cv + sign * k[partner] * sv;
+      }
+      qs[u][d] = qv;
+      ks[u][d] = kv * key_scale;
+    }
+    for (int idx = lane; idx < count * 16; idx += 64) {
+      const int u = idx / 16;
+      const int cc = idx - u * 16;
+      vs[u][cc] = v0 + cc < vdim
+                      ? p[static_cast<int64_t>(tb + u) * width + 2ll * heads * dim + static_cast<int64_t>(h) * vdim + v0 + cc]
+                      : 0.f;
+    }
+    __syncthreads();
+    for (int u = 0; u < count; ++u) {
+      const float vv = vs[u][c];
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) {
+        const int d = 4 * i + g;
+        if (d < dim) {
+          S[i] = fmaf(gamma, S[i], ks[u][d] * vv);
+          o = fmaf(S[i], qs[u][d], o);
+        }
+      }
+      o += __shfl_xor(o, 16, kWave);
+      o += __shfl_xor(o, 32, kWave);
+      if (g == 0 && column) out[static_cast<int64_t>(tb + u) * heads * vdim + static_cast<int64_t>(h) * vdim + v0 + c] = o;
+    }
+  }
+  float* dst = state + (static_cast<int64_t>(write_rows[entry]) * heads + h) * head_state;
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) {
+    const int d = 4 * i + g;
+    if (column && d < dim) dst[static_cast<int64_t>(d) * vdim + v0 + c] = S[i];
+  }
+}
+
+// out[t, h, :] = o / sqrt(mean(o^2) + eps) * silu(z), o = retained[t, h, :] (float32), z = the gate sums at
+// column gate_offset + h * vdim of p [tokens, width] (float32).  One wavefront per (token, head).
+template <typename T>
+__global__ __launch_bounds__(64) void retention_gate_kernel(const float* __restrict__ retained,
+                                                            const float* __restrict__ p, int width, int gate_offset,
+                                                            T* __restrict__ out, int heads, int vdim, float eps) {
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y;
+  const float* o = retained + (t * heads + h) * vdim;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < vdim; i += 64) ss += o[i] * o[i];
+  const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(vdim) + eps);
+  const float* z = p + t * width + gate_offset + static_cast<int64_t>(h) * vdim;
+  T* dst = out + (t * heads + h) * vdim;
+  for (int i = threadIdx.x; i < vdim; i += 64) {
+    const float zv = z[i];
+    dst[i] = from_f32<T>((o[i] * inv) * (zv / (1.0f + expf(-zv))));
+  }
+}
+
+}  // namespace mlr
+
+using namespace mlr;
+
+extern "C" {
+
+int mlr_add_normed(float* x, const void* y, int y_is_f32, int slices, const void* weight, int weight_is_f32, float eps,
+                   const void* next_weight, int next_is_f32, float next_eps, int mode, void* out, int dtype, int rows,
+                   int hidden, hipStream_t stream) {
+  MLR_REQUIRE(x && y && weight, "null pointer");
+  MLR_REQUIRE(rows > 0 && hidden > 0 && hidden <= 16384, "rows must be > 0 and hidden within 1..16384");
+  MLR_REQUIRE(slices >= 0 && (slices == 0 || y_is_f32), "partial sums are float32");
+  MLR_REQUIRE(mode >= 0 && mode <= 2 && (mode == 0 || out) && (mode != 1 || next_weight), "bad mode or missing output");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  MLR_REQUIRE(dtype == kBF16 || y_is_f32, "a float32 engine has float32 activations");
+  const size_t lds = static_cast<size_t>(hidden) * sizeof(float);
+  if (dtype == kF32)
+    add_normed_kernel<float><<<rows, 256, lds, stream>>>(x, y, y_is_f32, slices, rows, weight, weight_is_f32, eps,
+                                                         next_weight, next_is_f32, next_eps, mode,
+                                                         static_cast<float*>(out), hidden);
+  else
+    add_normed_kernel<bf16><<<rows, 256, lds, stream>>>(x, y, y_is_f32, slices, rows, weight, weight_is_f32, eps,
+                                                        next_weight, next_is_f32, next_eps, mode,
+                                                        static_cast<bf16*>(out), hidden);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_glu_clamped(const void* sums, int sums_is_f32, void* out, int dtype, int rows, int inter, float limit,
+                    float alpha, hipStream_t stream) {
+  MLR_REQUIRE(sums && out, "null pointer");
+  MLR_REQUIRE(rows > 0 && inter > 0 && limit > 0.f, "sizes and limit must be > 0");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  MLR_REQUIRE(dtype == kBF16 || sums_is_f32, "a float32 engine has float32 sums");
+  const int64_t total = static_cast<int64_t>(rows) * inter;
+  const int64_t blocks = (total + 255) / 256;
+  MLR_REQUIRE(blocks < (1ll << 31), "too many elements");
+  const unsigned grid = static_cast<unsigned>(blocks);
+  if (dtype == kF32)
+    glu_clamped_kernel<float, float><<<grid, 256, 0, stream>>>(static_cast<const float*>(sums), static_cast<float*>(out),
+                                                               rows, inter, limit, alpha);
+  else if (sums_is_f32)
+    glu_clamped_kernel<float, bf16><<<grid, 256, 0, stream>>>(static_cast<const float*>(sums), static_cast<bf16*>(out),
+                                                              rows, inter, limit, alpha);
+  else
+    glu_clamped_kernel<bf16, bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(sums), static_cast<bf16*>(out),
+                                                             rows, inter, limit, alpha);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_latent_prepare(const float* projected, int width, void* q_plain, void* q_latent, float* gate, const float* cos,
+                       const float* sin, int rotary_dims, const void* norm_weight, int weight_is_f32, float eps,
+                       const int* slots, void* key_pages, void* value_pages, int dtype, int tokens, int heads, int dim,
+                       int rot, int rank, int kernel_dim, int block_size, int num_pages, int own_cache, int gated,
+                       hipStream_t stream) {
+  MLR_REQUIRE(projected && q_plain && q_latent, "null pointer");
+  MLR_REQUIRE(tokens > 0 && heads > 0 && dim > 0 && rot > 0 && rank > 0, "sizes must be > 0");
+  MLR_REQUIRE(kernel_dim >= rank + rot, "the kernels' head size must hold latent and rotated part");
+  MLR_REQUIRE(rotary_dims >= 0 && rotary_dims % 2 == 0 && rotary_dims <= rot, "rotary_dims must be even and within rot");
+  MLR_REQUIRE(rotary_dims == 0 || (cos && sin), "a rotation needs cos and sin tables");
+  MLR_REQUIRE(width >= heads * (dim + rot) + (own_cache ? rank + rot : 0) + (gated ? heads : 0), "the projected rows are too narrow");
+  MLR_REQUIRE(!own_cache || (norm_weight && slots && key_pages && value_pages && block_size > 0 && num_pages > 0),
+              "a cache write needs the latent's norm weight, slots, pages and their sizes");
+  MLR_REQUIRE(!gated || gate, "a gated mixer needs room for its gates");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  if (dtype == kF32)
+    latent_prepare_kernel<float><<<tokens, 256, 0, stream>>>(
+        projected, width, static_cast<float*>(q_plain), static_cast<float*>(q_latent), gate, cos, sin, rotary_dims,
+        norm_weight, weight_is_f32, eps, slots, static_cast<float*>(key_pages), static_cast<float*>(value_pages), heads,
+        dim, rot, rank, kernel_dim, block_size, num_pages, own_cache, gated);
+  else
+    latent_prepare_kernel<bf16><<<tokens, 256, 0, stream>>>(
+        projected, width, static_cast<bf16*>(q_plain), static_cast<bf16*>(q_latent), gate, cos, sin, rotary_dims,
+        norm_weight, weight_is_f32, eps, slots, static_cast<bf16*>(key_pages), static_cast<bf16*>(value_pages), heads,
+        dim, rot, rank, kernel_dim, block_size, num_pages, own_cache, gated);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_heads_linear(const void* x, int64_t in_row, int in_stride, const void* w, void* out, int64_t out_row,
+                     int out_stride, const float* row_scale, int dtype, int tokens, int heads, int n, int k,
+                     hipStream_t stream) {
+  MLR_REQUIRE(x && w && out, "null pointer");
+  MLR_REQUIRE(tokens > 0 && heads > 0 && n > 0 && k > 0, "sizes must be > 0");
+  MLR_REQUIRE(in_stride >= k && in_row >= static_cast<int64_t>(heads) * in_stride, "the input rows do not hold every head's k values");
+  MLR_REQUIRE(out_stride >= n && out_row >= static_cast<int64_t>(heads) * out_stride, "the output rows do not hold every head's n values");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  dim3 grid((n + 63) / 64, (tokens + 63) / 64, heads);
+  MLR_REQUIRE(grid.y < 65536u && grid.z < 65536u, "too many rows or heads for one launch");
+  if (dtype == kF32)
+    heads_linear_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(x), in_row, in_stride,
+                                                         static_cast<const float*>(w), static_cast<float*>(out), out_row,
+                                                         out_stride, row_scale, heads, tokens, n, k);
+  else
+    heads_linear_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(x), in_row, in_stride,
+                                                        static_cast<const bf16*>(w), static_cast<bf16*>(out), out_row,
+                                                        out_stride, row_scale, heads, tokens, n, k);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_retention_scan(const float* projected, int width, float* state, int state_rows, const int* read_rows,
+                       const int* write_rows, const int* cu_q, const int* q_starts, const float* decay,
+                       const float* cos, const float* sin, int rotary_dims, float key_scale, float* out, int entries,
+                       int heads, int dim, int vdim, hipStream_t stream) {
+  MLR_REQUIRE(projected && state && read_rows && write_rows && cu_q && q_starts && decay && out, "null pointer");
+  MLR_REQUIRE(entries > 0 && heads > 0 && dim > 0 && vdim > 0 && state_rows > 0, "sizes must be > 0");
+  MLR_REQUIRE(dim <= 256, "a head's state has up to 256 rows");
+  MLR_REQUIRE(width >= 2 * heads * dim + heads * vdim, "the projected rows are too narrow");
+  MLR_REQUIRE(rotary_dims >= 0 && rotary_dims % 2 == 0 && rotary_dims <= dim, "rotary_dims must be even and within dim");
+  MLR_REQUIRE(rotary_dims == 0 || (cos && sin), "a rotation needs cos and sin tables");
+  dim3 grid(entries, heads, (vdim + 15) / 16);
+  MLR_REQUIRE(grid.y < 65536u && grid.z < 65536u, "too many heads or columns for one launch");
+#define MLR_SCAN(dpl)                                                                                              \
+  retention_scan_kernel<dpl><<<grid, 64, 0, stream>>>(projected, width, state, read_rows, write_rows, cu_q, q_starts, \
+                                                      decay, cos, sin, rotary_dims, key_scale, out, heads, dim, vdim)
+  if (dim <= 16)
+    MLR_SCAN(4);
+  else if (dim <= 32)
+    MLR_SCAN(8);
+  else if (dim <= 64)
+    MLR_SCAN(16);
+  else if (dim <= 128)
+    MLR_SCAN(32);
+  else
+    MLR_SCAN(64);
+#undef MLR_SCAN
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_retention_gate(const float* retained, const float* projected, int width, int gate_offset, void* out, int dtype,
+                       int tokens, int heads, int vdim, float eps, hipStream_t stream) {
+  MLR_REQUIRE(retained && projected && out, "null pointer");
+  MLR_REQUIRE(tokens > 0 && heads > 0 && heads < 65536 && vdim > 0, "sizes must be > 0");
+  MLR_REQUIRE(gate_offset >= 0 && width >= gate_offset + heads * vdim, "the projected rows do not hold the gate");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  dim3 grid(tokens, heads);
+  if (dtype == kF32)
+    retention_gate_kernel<float><<<grid, 64, 0, stream>>>(retained, projected, width, gate_offset,
+                                                          static_cast<float*>(out), heads, vdim, eps);
+  else
+    retention_gate_kernel<bf16><<<grid, 64, 0, stream>>>(retained, projected, width, gate_offset,
+                                                         static_cast<bf16*>(out), heads, vdim, eps);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

@@ -65,6 +65,7 @@ CORE = Module(
         "gemm_stream.hip",
         "attention_simple.hip",
         "moe.hip",
+        "mixers.hip",
         "sampling.hip",
     ),
 )

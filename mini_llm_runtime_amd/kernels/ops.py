@@ -18,7 +18,7 @@ from typing import Any, Optional, Sequence, Union
 import torch
 
 from . import build
-from .pending import PendingLinear, PendingMerge, PendingNorm, PendingScale
+from .pending import NormedDelta, PendingLinear, PendingMerge, PendingNorm, PendingScale
 from .tuning import KernelTuning
 
 _VP = ctypes.c_void_p
@@ -28,13 +28,22 @@ _F = ctypes.c_float
 
 _SIGNATURES = {
     "mlr_version": ([], _I),
-    "mlr_embedding": ([_VP, _I, _VP, _VP, _I, _I, _I, _VP], _I),
+    "mlr_embedding": ([_VP, _I, _VP, _VP, _I, _I, _I, _I, _VP], _I),
+    "mlr_add_normed": ([_VP, _VP, _I, _I, _VP, _I, _F, _VP, _I, _F, _I, _VP, _I, _I, _I, _VP], _I),
+    "mlr_glu_clamped": ([_VP, _I, _VP, _I, _I, _I, _F, _F, _VP], _I),
+    "mlr_latent_prepare": (
+        [_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _VP, _I, _F, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP],
+        _I,
+    ),
+    "mlr_heads_linear": ([_VP, _I64, _I, _VP, _VP, _I64, _I, _VP, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_retention_scan": ([_VP, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _F, _VP, _I, _I, _I, _I, _VP], _I),
+    "mlr_retention_gate": ([_VP, _VP, _I, _I, _VP, _I, _I, _I, _I, _F, _VP], _I),
     "mlr_rmsnorm": ([_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _I, _F, _VP], _I),
     "mlr_add": ([_VP, _VP, _I, _I64, _VP], _I),
     "mlr_scale_softcap": ([_VP, _F, _F, _I64, _VP], _I),
     "mlr_gather_rows": ([_VP, _VP, _VP, _I, _I64, _I, _I, _VP], _I),
     "mlr_silu_mul": ([_VP, _VP, _I, _I, _I, _VP], _I),
-    "mlr_rope_table": ([_VP, _VP, _VP, _VP, _I, _I, _VP], _I),
+    "mlr_rope_table": ([_VP, _VP, _VP, _VP, _I, _I, _F, _VP], _I),
     "mlr_rope_kv_write": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_qkv_finish": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP], _I),
@@ -62,7 +71,7 @@ _SIGNATURES = {
     ),
     "mlr_gemm_merge_fused_bf16": ([_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I, _VP, _I, _I, _I, _I, _VP], _I),
     "mlr_paged_attention_simple": (
-        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _VP],
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _VP, _VP],
         _I,
     ),
     "mlr_sample": ([_VP, _VP, _VP, _VP, _VP, _I, _I, _VP], _I),
@@ -72,19 +81,19 @@ _SIGNATURES = {
     "mlr_attention_wide_tile": ([], _I),
     "mlr_attention_decode_scratch": ([_I, _I, _I], _I64),
     "mlr_attention_decode": (
-        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _VP],
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _VP, _VP],
         _I,
     ),
-    "mlr_attention_decode_merge": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_attention_decode_merge": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP], _I),
     "mlr_attention_prefill_scratch": ([_I, _I, _I, _I], _I64),
     "mlr_attention_prefill": (
-        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _I, _I, _VP, _VP],
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _I, _I, _VP, _VP, _VP],
         _I,
     ),
 }
 
 # what `linear` may do to its sums before it stores them (the entry points' `swiglu` argument)
-_EPILOGUES = {None: 0, "swiglu": 1, "relu2": 2, "sigmoid": 3}
+_EPILOGUES = {None: 0, "swiglu": 1, "relu2": 2, "sigmoid": 3, "gelu_tanh": 4}
 
 from .plans import PAGED_ATTENTION, QUERY_TILE, WIDE_QUERY_TILE, attention_plan, query_tiles  # noqa: F401
 
@@ -216,13 +225,17 @@ class HipOps:
         return torch.empty(tuple(shape), dtype=dtype, device=self.device)
 
     # ---- residual stream --------------------------------------------------------------------
-    def embedding(self, table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    def embedding(self, table: torch.Tensor, ids: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        """table[ids] as float32 (the residual stream), or in `out_dtype` = the engine's dtype."""
         self._check(table, "embedding table", self.dtype, (None, None))
         self._check(ids, "token ids", torch.int32, (None,))
+        out_dtype = out_dtype or torch.float32
+        if out_dtype not in (torch.float32, self.dtype):
+            raise KernelError(f"embedding output must be float32 or {self.dtype}")
         vocab, hidden = table.shape
-        out = self._empty((ids.shape[0], hidden), torch.float32)
+        out = self._empty((ids.shape[0], hidden), out_dtype)
         self._call(
-            "mlr_embedding", self._ptr(table), self.code, self._ptr(ids), self._ptr(out),
+            "mlr_embedding", self._ptr(table), self.code, self._ptr(ids), self._ptr(out), int(out_dtype == torch.float32),
             ids.shape[0], hidden, vocab, self._stream(),
         )
         return out
@@ -233,6 +246,8 @@ class HipOps:
         """x (float32 residual stream [rows, hidden]) += delta in place, then the RMSNorm of x
         in the engine's dtype.  delta: [rows, hidden] in the engine's dtype, or a float32 stack
         [S, rows, hidden] of partial sums (see `linear`), or None."""
+        if isinstance(delta, NormedDelta):  # one kernel: the normed addition and this norm
+            return self.add_normed(x, delta.y, delta.weight, delta.eps, next_weight=weight, next_eps=eps)
         self._check(x, "residual stream", torch.float32, (None, None))
         rows, hidden = x.shape
         self._check(weight, "norm weight", (torch.float32, self.dtype), (hidden,))
@@ -248,6 +263,48 @@ class HipOps:
         self._call(
             "mlr_rmsnorm", self._ptr(x), self._ptr(plain), self._ptr(partial), slices, self._ptr(weight),
             int(weight.dtype == torch.float32), self._ptr(out), self.code, rows, hidden, float(eps), self._stream(),
+        )
+        return out
+
+    def add_normed(
+        self,
+        x: torch.Tensor,
+        y,
+        weight: torch.Tensor,
+        eps: float,
+        next_weight: Optional[torch.Tensor] = None,
+        next_eps: float = 0.0,
+        cast: bool = False,
+    ) -> Optional[torch.Tensor]:
+        """x (float32 residual stream [rows, hidden], in place) += weight * y * rsqrt(mean(y^2) + eps): a part's
+        output that enters the stream through a norm of its own.  y: [rows, hidden] in the engine's dtype or
+        float32, a float32 stack [S, rows, hidden] whose sum it is, or a product that has not run.  The same
+        kernel then makes what reads the stream next: with `next_weight` the RMSNorm of the new x (weight,
+        `next_eps`), with `cast` x itself, both in the engine's dtype; else nothing is returned."""
+        self._check(x, "residual stream", torch.float32, (None, None))
+        rows, hidden = x.shape
+        y = self.settle(y)
+        slices = 0
+        if y.dim() == 3:
+            self._check(y, "partial sums", torch.float32, (None, rows, hidden))
+            slices = y.shape[0]
+        else:
+            self._check(y, "sublayer output", (torch.float32, self.dtype), (rows, hidden))
+        self._check(weight, "norm weight", (torch.float32, self.dtype), (hidden,))
+        mode = 0
+        out = None
+        if next_weight is not None:
+            self._check(next_weight, "next norm weight", (torch.float32, self.dtype), (hidden,))
+            mode = 1
+        elif cast:
+            mode = 2
+        if mode:
+            out = self._empty((rows, hidden), self.dtype)
+        self._call(
+            "mlr_add_normed", self._ptr(x), self._ptr(y), int(y.dtype == torch.float32), slices, self._ptr(weight),
+            int(weight.dtype == torch.float32), float(eps), self._ptr(next_weight),
+            int(next_weight is not None and next_weight.dtype == torch.float32), float(next_eps), mode, self._ptr(out),
+            self.code, rows, hidden, self._stream(),
         )
         return out
 
@@ -271,6 +328,8 @@ class HipOps:
         the same kernels whether it was chosen or all rows were taken."""
         if isinstance(x, PendingLinear):
             return PendingLinear(self.gather_rows(self.settle(x.x), rows), x.weight, x.bias)
+        if isinstance(x, NormedDelta):  # the norm is per row: it commutes with the choice of rows
+            return NormedDelta(self.gather_rows(x.y, rows), x.weight, x.eps)
         x = self.settle(x)
         self._check(x, "rows source", (torch.float32, torch.bfloat16))
         if x.dim() not in (2, 3):
@@ -298,6 +357,8 @@ class HipOps:
     def defer_norm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, delta: Optional[torch.Tensor]):
         """The norm of `rmsnorm` as a `PendingNorm` when the product behind it could compute it
         in its own kernel (bfloat16, few tokens, a narrow model); else None."""
+        if isinstance(delta, NormedDelta):
+            return None  # the norm kernel that adds a normed delta makes the activations itself
         if isinstance(delta, PendingLinear):
             return self._finish_stream(x, weight, float(eps), delta)  # None: the caller's norm kernel settles it
         if not (self.tuning.fuse_norm and self.dtype == torch.bfloat16 and x.dim() == 2):
@@ -323,11 +384,16 @@ class HipOps:
             return h.value
         if isinstance(h, PendingLinear):
             return self.linear(h.x, h.weight, h.bias, partial_sums=True)
+        if isinstance(h, NormedDelta):  # what it adds to the stream, float32
+            y = self.settle(h.y)
+            added = torch.zeros(y.shape[-2:], dtype=torch.float32, device=self.device)
+            self.add_normed(added, y, h.weight, h.eps)
+            return added
         if isinstance(h, PendingMerge):
             out = self._empty((h.tokens, h.heads * h.head_dim), self.dtype)
             self._call(
                 "mlr_attention_decode_merge", self._ptr(h.partial), self._ptr(h.cu_q), self._ptr(h.context_lens),
-                self._ptr(out), h.tokens, h.heads, h.window, 0, h.part, h.splits, self._stream(), lib=h.library,
+                self._ptr(out), h.tokens, h.heads, h.window, 0, h.part, h.splits, _VP(None), self._stream(), lib=h.library,
             )
             return out
         return h
@@ -559,7 +625,9 @@ class HipOps:
         return out
 
     # ---- positions and cache ---------------------------------------------------------------------
-    def rope_table(self, positions: torch.Tensor, inv_freq: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    def rope_table(
+        self, positions: torch.Tensor, inv_freq: torch.Tensor, amplitude: float = 1.0
+    ) -> tuple[torch.Tensor, torch.Tensor]:
         self._check(positions, "positions", torch.int32, (None,))
         self._check(inv_freq, "inverse frequencies", torch.float64, (None,))
         tokens, half = positions.shape[0], inv_freq.shape[0]
@@ -567,7 +635,7 @@ class HipOps:
         sin = self._empty((tokens, half), torch.float32)
         self._call(
             "mlr_rope_table", self._ptr(positions), self._ptr(inv_freq), self._ptr(cos), self._ptr(sin),
-            tokens, half, self._stream(),
+            tokens, half, float(amplitude), self._stream(),
         )
         return cos, sin
 
@@ -779,8 +847,12 @@ class HipOps:
         defer_merge: bool = False,
         plan: Any = None,
         chunk: Optional[int] = None,
+        sinks: Optional[torch.Tensor] = None,
     ):
         """Causal attention of the step's tokens over their requests' pages.
+
+        sinks: float32 [num_heads]; the softmax's denominator of head h then also holds exp(sinks[h]), a
+        term with no key and no value (not scaled).
 
         window / chunk: which of the keys 0..p a query at position p sees: with a window the last
         `window` of them, with a chunked mask those from floor(p / chunk) * chunk on; at most one of
@@ -818,6 +890,8 @@ class HipOps:
         if chunk is not None and (chunk <= 0 or window):
             raise KernelError("a chunked mask has a size > 0 and no window beside it")
         chunk = int(chunk or 0)
+        if sinks is not None:
+            self._check(sinks, "sinks", torch.float32, (num_heads,))
         out = self._empty((tokens, num_heads * head_dim), self.dtype)
         width = block_table.shape[1]
         use_mfma = (
@@ -842,7 +916,7 @@ class HipOps:
                 "mlr_paged_attention_simple", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
                 self._ptr(block_table), width, self._ptr(ctx.token_entry), self._ptr(ctx.positions),
                 self._ptr(out), self.code, tokens, entries, num_heads, num_kv_heads, head_dim, block_size,
-                num_pages, float(scale), int(window or 0), chunk, self._stream(),
+                num_pages, float(scale), int(window or 0), chunk, self._ptr(sinks), self._stream(),
             )
             return out
         self._check(ctx.cu_q, "cu_q", torch.int32, (entries + 1,))
@@ -866,13 +940,13 @@ class HipOps:
                 partial = self._empty((lib.mlr_attention_decode_scratch(entries, num_heads, splits),), torch.float32)
             leave_unmerged = (
                 defer_merge and self.tuning.fuse_merge and not num_tiles and num_decode == entries == tokens
-                and 1 < splits <= 64 and tokens <= self.FUSED_TOKENS and not chunk
+                and 1 < splits <= 64 and tokens <= self.FUSED_TOKENS and not chunk and sinks is None
             )
             self._call(
                 "mlr_attention_decode", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
                 self._ptr(block_table), width, self._ptr(ctx.cu_q), self._ptr(ctx.context_lens), self._ptr(out),
                 self._ptr(partial), entries, num_heads, num_kv_heads, block_size, num_pages, float(scale),
-                int(window or 0), chunk, part, splits, int(not leave_unmerged), self._stream(), lib=lib,
+                int(window or 0), chunk, part, splits, int(not leave_unmerged), self._ptr(sinks), self._stream(), lib=lib,
             )
             if leave_unmerged:
                 return PendingMerge(
@@ -909,8 +983,170 @@ class HipOps:
                 "mlr_attention_prefill", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
                 self._ptr(block_table), width, self._ptr(tiles), num_tiles, wide, self._ptr(ctx.cu_q),
                 self._ptr(ctx.context_lens), self._ptr(out), num_heads, num_kv_heads, block_size, num_pages,
-                float(scale), int(window or 0), chunk, key_runs, self._ptr(partial), self._stream(), lib=lib,
+                float(scale), int(window or 0), chunk, key_runs, self._ptr(partial), self._ptr(sinks), self._stream(),
+                lib=lib,
             )
+        return out
+
+    # ---- other mixers and feed-forwards ----------------------------------------------------------------
+    def glu_clamped(self, sums: torch.Tensor, limit: float, alpha: float = 1.702) -> torch.Tensor:
+        """sums [rows, 2 * inter] (gate sums, then up sums; float32 or the engine's dtype) ->
+        g * sigmoid(alpha * g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit), [rows, inter]."""
+        self._check(sums, "gate and up sums", (torch.float32, self.dtype), (None, None))
+        rows, width = sums.shape
+        if width % 2:
+            raise KernelError("gate and up sums must have an even width")
+        out = self._empty((rows, width // 2), self.dtype)
+        self._call(
+            "mlr_glu_clamped", self._ptr(sums), int(sums.dtype == torch.float32), self._ptr(out), self.code, rows,
+            width // 2, float(limit), float(alpha), self._stream(),
+        )
+        return out
+
+    def latent_prepare(
+        self,
+        projected: torch.Tensor,
+        *,
+        heads: int,
+        head_dim: int,
+        rot_dim: int,
+        kv_rank: int,
+        own_cache: bool,
+        gated: bool,
+        norm_weight: Optional[torch.Tensor],
+        eps: float,
+        rotation: Optional[tuple[torch.Tensor, torch.Tensor, int]],
+        slot_mapping: torch.Tensor,
+        key_pages: torch.Tensor,
+        value_pages: torch.Tensor,
+        block_size: int,
+        kernel_dim: int,
+    ):
+        """From a latent-attention layer's input sums (float32 [T, heads * (head_dim + rot_dim) (+ kv_rank +
+        rot_dim) (+ heads)]: queries, own latent and shared key part, gate logits) to what its kernels take:
+        (unrotated query parts [T, heads * head_dim]; latent queries [T, heads * kernel_dim] whose columns
+        kv_rank .. kv_rank + rot_dim hold the rotated query parts and whose first kv_rank are left to
+        `heads_linear`; gates sigmoid(logit), float32 [T, heads], or None).  With `own_cache` the normed latent
+        and the rotated key part go into the pages: key rows [latent ; key part ; 0], values [latent ; 0]."""
+        self._check(projected, "projected input", torch.float32, (None, None))
+        tokens, width = projected.shape
+        cos = sin = None
+        rotary = 0
+        if rotation is not None:
+            cos, sin, rotary = rotation
+            self._check(cos, "rotary cos", torch.float32, (tokens, rotary // 2))
+            self._check(sin, "rotary sin", torch.float32, (tokens, rotary // 2))
+        num_pages = 0
+        if own_cache:
+            num_pages = self._check_pages(key_pages, value_pages, 1, kernel_dim, block_size)
+            self._check(slot_mapping, "slot mapping", torch.int32, (tokens,))
+            self._check(norm_weight, "latent norm weight", (torch.float32, self.dtype), (kv_rank,))
+        q_plain = self._empty((tokens, heads * head_dim), self.dtype)
+        q_latent = self._empty((tokens, heads * kernel_dim), self.dtype)
+        gate = self._empty((tokens, heads), torch.float32) if gated else None
+        self._call(
+            "mlr_latent_prepare", self._ptr(projected), width, self._ptr(q_plain), self._ptr(q_latent), self._ptr(gate),
+            self._ptr(cos), self._ptr(sin), int(rotary), self._ptr(norm_weight if own_cache else None),
+            int(own_cache and norm_weight.dtype == torch.float32), float(eps),
+            self._ptr(slot_mapping if own_cache else None), self._ptr(key_pages if own_cache else None),
+            self._ptr(value_pages if own_cache else None), self.code, tokens, heads, head_dim, rot_dim, kv_rank,
+            kernel_dim, block_size, num_pages, int(own_cache), int(gated), self._stream(),
+        )
+        return q_plain, q_latent, gate
+
+    def heads_linear(
+        self,
+        x: torch.Tensor,
+        weight: torch.Tensor,
+        *,
+        in_stride: int,
+        out: Optional[torch.Tensor] = None,
+        out_stride: Optional[int] = None,
+        row_scale: Optional[torch.Tensor] = None,
+    ) -> torch.Tensor:
+        """One small matrix per head: y[t, h, :] = weight[h] x[t, h, :k] for weight [heads, n, k] and x [T, heads
+        * in_stride] (head h's input starts at column h * in_stride), times row_scale[t, h] (float32) if given.
+        Returns [T, heads * n], or writes head h's result to columns h * out_stride .. + n of `out`."""
+        self._check(weight, "per-head weights", self.dtype, (None, None, None))
+        heads, n, k = weight.shape
+        self._check(x, "per-head input", self.dtype, (None, None))
+        tokens = x.shape[0]
+        if in_stride < k or x.shape[1] < heads * in_stride:
+            raise KernelError("the input rows do not hold every head's values")
+        if out is None:
+            out_stride = n
+            out = self._empty((tokens, heads * n), self.dtype)
+        else:
+            self._check(out, "per-head output", self.dtype, (tokens, None))
+            if out_stride is None or out_stride < n or out.shape[1] < heads * out_stride:
+                raise KernelError("the output rows do not hold every head's values")
+        if row_scale is not None:
+            self._check(row_scale, "row scale", torch.float32, (tokens, heads))
+        self._call(
+            "mlr_heads_linear", self._ptr(x), x.shape[1], int(in_stride), self._ptr(weight), self._ptr(out), out.shape[1],
+            int(out_stride), self._ptr(row_scale), self.code, tokens, heads, n, k, self._stream(),
+        )
+        return out
+
+    def retention_scan(
+        self,
+        projected: torch.Tensor,
+        state: torch.Tensor,
+        read_rows: torch.Tensor,
+        write_rows: torch.Tensor,
+        ctx: Any,
+        *,
+        heads: int,
+        head_dim: int,
+        value_dim: int,
+        decay: torch.Tensor,
+        key_scale: float,
+        rotation: Optional[tuple[torch.Tensor, torch.Tensor, int]],
+    ) -> torch.Tensor:
+        """Retention of the step's tokens, every entry's in order: S = decay_h S + k v^T, o = S^T q per head,
+        from the state in row read_rows[entry] of `state` [rows, heads, head_dim, value_dim] (zeros where the
+        entry starts its request) to row write_rows[entry].  `projected` (float32 [T, >= 2 * heads * head_dim +
+        heads * value_dim]) holds q, k and v; q and k are rotated and k scaled by `key_scale` here, in 32-bit.
+        Returns o, float32 [T, heads * value_dim]."""
+        self._check(projected, "projected input", torch.float32, (None, None))
+        tokens, width = projected.shape
+        entries = ctx.num_entries
+        self._check(state, "retention state", torch.float32, (None, heads, head_dim, value_dim))
+        self._check(read_rows, "state rows to read", torch.int32, (entries,))
+        self._check(write_rows, "state rows to write", torch.int32, (entries,))
+        self._check(ctx.cu_q, "cu_q", torch.int32, (entries + 1,))
+        self._check(ctx.q_starts, "q_starts", torch.int32, (entries,))
+        self._check(decay, "decays", torch.float32, (heads,))
+        cos = sin = None
+        rotary = 0
+        if rotation is not None:
+            cos, sin, rotary = rotation
+            self._check(cos, "rotary cos", torch.float32, (tokens, rotary // 2))
+            self._check(sin, "rotary sin", torch.float32, (tokens, rotary // 2))
+        out = self._empty((tokens, heads * value_dim), torch.float32)
+        self._call(
+            "mlr_retention_scan", self._ptr(projected), width, self._ptr(state), state.shape[0], self._ptr(read_rows),
+            self._ptr(write_rows), self._ptr(ctx.cu_q), self._ptr(ctx.q_starts), self._ptr(decay), self._ptr(cos),
+            self._ptr(sin), int(rotary), float(key_scale), self._ptr(out), entries, heads, head_dim, value_dim,
+            self._stream(),
+        )
+        return out
+
+    def retention_gate(
+        self, retained: torch.Tensor, projected: torch.Tensor, *, heads: int, value_dim: int, gate_offset: int, eps: float
+    ) -> torch.Tensor:
+        """Every head's retained[t, h, :] divided by its root mean square (eps inside the root), times silu of
+        the gate sums in columns gate_offset .. of `projected`; [T, heads * value_dim] in the engine's dtype."""
+        self._check(projected, "projected input", torch.float32, (None, None))
+        tokens, width = projected.shape
+        self._check(retained, "retained", torch.float32, (tokens, heads * value_dim))
+        if gate_offset < 0 or gate_offset + heads * value_dim > width:
+            raise KernelError("the projected rows do not hold the gate")
+        out = self._empty((tokens, heads * value_dim), self.dtype)
+        self._call(
+            "mlr_retention_gate", self._ptr(retained), self._ptr(projected), width, int(gate_offset), self._ptr(out),
+            self.code, tokens, heads, value_dim, float(eps), self._stream(),
+        )
         return out
 
     # ---- routed experts --------------------------------------------------------------------------------
