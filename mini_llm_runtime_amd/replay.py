@@ -4,7 +4,7 @@ cache manager and kernels, the ones generation uses; it has no forward pass,
 cache or loader of its own.
 
     bin/trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
-                  [--block-size 16] [--max-live 8] [--layers]
+                  [--block-size 16] [--max-live 4] [--layers]
 
 Steps come on standard input, one JSON object a line:
 
@@ -32,7 +32,7 @@ from typing import Any, Optional, Sequence, TextIO
 
 
 PAGE_TOKENS = 16  # default tokens per page of the replay pool
-MAX_LIVE = 8  # default number of request slots
+MAX_LIVE = 4  # default number of request slots (state banks and block table rows are made for this many)
 
 
 def parse_args(argv: Optional[Sequence[str]] = None) -> argparse.Namespace:
