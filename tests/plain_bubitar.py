@@ -5,13 +5,38 @@ engine and is what the engine's parts, kernels and schedules are compared with.
 Notation: x is the residual stream [T, width]; h a normed input; positions count from 0.
 A model is a dict `config` (the keys of the design's config.json) and a dict `weights`
 (tensor name -> tensor, names as in the design's checkpoints).
+
+`rounded()` switches every matrix product to operands and results rounded to bfloat16 (everything
+else stays float64): what rounding alone does to a row of logits, which is the yardstick for a
+bfloat16 engine where a model is ill-conditioned (a sublayer's output near zero before its norm).
 """
 
 from __future__ import annotations
 
+import contextlib
 import math
 
 import torch
+
+_ROUND = [False]
+
+
+@contextlib.contextmanager
+def rounded():
+    _ROUND.append(True)
+    try:
+        yield
+    finally:
+        _ROUND.pop()
+
+
+def _r(t: torch.Tensor) -> torch.Tensor:
+    return t.to(torch.bfloat16).double() if _ROUND[-1] else t
+
+
+def mm(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """a @ w^T, the one place where products happen."""
+    return _r(_r(a) @ w.T)
 
 
 def rms_norm(x: torch.Tensor, w, eps: float) -> torch.Tensor:
@@ -56,7 +81,7 @@ def rotate(x: torch.Tensor, positions: torch.Tensor, rot: dict) -> torch.Tensor:
 def latent_cache(h: torch.Tensor, w: dict, m: dict, eps: float, positions: torch.Tensor):
     """(latents [T, kv_rank], rotated shared key part [T, rot_dim]) that a layer with `dkv` makes."""
     R = m["kv_rank"]
-    down = h @ w["dkv"].T
+    down = mm(h, w["dkv"])
     return rms_norm(down[:, :R], w["dkv.norm"], eps), rotate(down[:, None, R:], positions, m["rot"])[:, 0]
 
 
@@ -65,10 +90,10 @@ def latent_attention(h: torch.Tensor, w: dict, m: dict, cache, positions: torch.
     T = h.shape[0]
     H, d, r, dv = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
     latent, shared = cache
-    q = (h @ w["q"].T).view(T, H, d + r)
+    q = mm(h, w["q"]).view(T, H, d + r)
     q_plain, q_turned = q[..., :d], rotate(q[..., d:], positions, m["rot"])
-    k_plain = (latent @ w["uk"].T).view(T, H, d)
-    v = (latent @ w["uv"].T).view(T, H, dv)
+    k_plain = mm(latent, w["uk"]).view(T, H, d)
+    v = mm(latent, w["uv"]).view(T, H, dv)
     scores = (torch.einsum("ihd,jhd->hij", q_plain, k_plain) + torch.einsum("ihr,jr->hij", q_turned, shared)) * m["scale"]
     seen = positions[None, :] <= positions[:, None]
     scores = scores.masked_fill(~seen, -math.inf)
@@ -78,16 +103,16 @@ def latent_attention(h: torch.Tensor, w: dict, m: dict, cache, positions: torch.
     e = torch.exp(scores - top[..., None])
     weights = e / (e.sum(-1) + torch.exp(sink[:, None] - top))[..., None]
     out = torch.einsum("hij,jhv->ihv", weights, v)
-    out = out * torch.sigmoid(h @ w["g"].T)[..., None]  # one gate per head and token
-    return out.reshape(T, H * dv) @ w["o"].T
+    out = out * torch.sigmoid(mm(h, w["g"]))[..., None]  # one gate per head and token
+    return mm(out.reshape(T, H * dv), w["o"])
 
 
 def retention(h: torch.Tensor, w: dict, m: dict, eps: float, positions: torch.Tensor) -> torch.Tensor:
     T = h.shape[0]
     H, d, dv = m["heads"], m["dim"], m["vdim"]
-    q = rotate((h @ w["q"].T).view(T, H, d), positions, m["rot"])
-    k = rotate((h @ w["k"].T).view(T, H, d), positions, m["rot"]) * d**-0.5
-    v = (h @ w["v"].T).view(T, H, dv)
+    q = rotate(mm(h, w["q"]).view(T, H, d), positions, m["rot"])
+    k = rotate(mm(h, w["k"]).view(T, H, d), positions, m["rot"]) * d**-0.5
+    v = mm(h, w["v"]).view(T, H, dv)
     out = torch.zeros(T, H, dv, dtype=h.dtype)
     for head in range(H):
         state = torch.zeros(d, dv, dtype=h.dtype)
@@ -95,20 +120,20 @@ def retention(h: torch.Tensor, w: dict, m: dict, eps: float, positions: torch.Te
             state = m["decay"][head] * state + torch.outer(k[t, head], v[t, head])
             out[t, head] = state.T @ q[t, head]
     out = rms_norm(out, None, eps).reshape(T, H * dv)
-    z = h @ w["g"].T
-    return (out * (z * torch.sigmoid(z))) @ w["o"].T
+    z = mm(h, w["g"])
+    return mm(out * (z * torch.sigmoid(z)), w["o"])
 
 
 def clamped_feed_forward(h: torch.Tensor, w: dict, m: dict) -> torch.Tensor:
     limit = m["limit"]
-    g = torch.clamp(h @ w["gate"].T + w["gate.b"], max=limit)
-    u = torch.clamp(h @ w["up"].T + w["up.b"], -limit, limit)
-    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ w["down"].T + w["down.b"]
+    g = torch.clamp(mm(h, w["gate"]) + w["gate.b"], max=limit)
+    u = torch.clamp(mm(h, w["up"]) + w["up.b"], -limit, limit)
+    return mm(g * torch.sigmoid(1.702 * g) * (u + 1.0), w["down"]) + w["down.b"]
 
 
 def token_input(x: torch.Tensor, rows: torch.Tensor, w: dict) -> torch.Tensor:
     """rows: the layer's columns of the shared table at the tokens, [T, side dim]."""
-    return (gelu_tanh(x @ w["gate"].T) * rows) @ w["proj"].T
+    return mm(gelu_tanh(mm(x, w["gate"])) * rows, w["proj"])
 
 
 def _sub(weights: dict, prefix: str) -> dict:
@@ -143,4 +168,4 @@ def forward(config: dict, weights: dict, tokens, layer_outputs=None) -> torch.Te
         x = x + rms_norm(token_input(x, rows, sw), sw["norm"], eps)
         if layer_outputs is not None:
             layer_outputs.append(x.clone())
-    return rms_norm(x, weights["final.norm"].double(), eps) @ weights["head"].double().T
+    return _r(rms_norm(x, weights["final.norm"].double(), eps)) @ weights["head"].double().T

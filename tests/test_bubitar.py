@@ -189,18 +189,25 @@ GPU_CASES = [
 ]
 
 
-def _compare(got, requests, weights, cfg, dtype, f32_bound=1e-4, row_bound=0.12, together=2.5e-2):
+def _compare(got, requests, weights, cfg, dtype, f32_bound=1e-4, row_bound=6e-2, together=2.5e-2):
     """float32: every value within 1e-4 of the logits' size.  bfloat16: all rows together within 2.5 %
-    (relative L2) and every single row within 12 %: these weights make scores of ten and more, so one
-    rounding of a query or a cached latent moves a score by a tenth, and where a sink and a few keys
-    share the weight (the first positions of a request) that moves the balance between the heads by
-    several percent, which the norm behind every sublayer passes on at full size.  The same rows stand
-    out under every schedule; a wrong key, page, slot or state changes a row by half and more."""
+    (relative L2); every row within 6 %, but for a few (one in twenty) that may be off by up to 4 times what
+    rounding alone does to the worst row of their request (the plain implementation with its products
+    rounded to bfloat16).  A sublayer's output passes a norm before it is added, so where that output is
+    near zero, or where a sink and one or two keys share the weight, every rounding moves the row by a
+    percent, in the plain implementation as in the engine, and the worst row of hundreds is one where
+    they all push the same way: the same rows stand out under every schedule.  A wrong key, page, slot or
+    state changes a row by half and more, and most rows."""
     assert got, "no logits came back"
     num = den = 0.0
+    loose = rows = 0
     for rid, toks in requests.items():
         ref = plain.forward(cfg, weights, toks)
         size = float(ref.pow(2).mean().sqrt())
+        if dtype != torch.float32:
+            with plain.rounded():
+                coarse = plain.forward(cfg, weights, toks)
+            alone = (coarse - ref).pow(2).sum(-1).sqrt() / ref.pow(2).sum(-1).sqrt()
         for pos in range(len(toks)):
             row = got[(rid, pos)].double()
             assert torch.isfinite(row).all(), f"{rid}:{pos} is not finite"
@@ -208,11 +215,16 @@ def _compare(got, requests, weights, cfg, dtype, f32_bound=1e-4, row_bound=0.12,
             if dtype == torch.float32:
                 assert float(diff.abs().max()) < f32_bound * size, f"{rid}:{pos}: off by {float(diff.abs().max()):.3e}"
                 continue
+            rows += 1
             rel = float(diff.pow(2).sum().sqrt() / ref[pos].pow(2).sum().sqrt())
-            assert rel < row_bound, f"{rid}:{pos}: relative error {rel:.3e}"
+            if rel >= row_bound:
+                loose += 1
+                assert rel < 4.0 * float(alone.max()), f"{rid}:{pos}: relative error {rel:.3e}, rounding alone up to {float(alone.max()):.3e}"
+                continue
             num += float(diff.pow(2).sum())
             den += float(ref[pos].pow(2).sum())
     if dtype != torch.float32:
+        assert loose <= 0.05 * rows + 1, f"{loose} of {rows} rows are ill-conditioned: the test's model is no yardstick"
         assert (num / den) ** 0.5 < together, f"relative error of all rows {(num / den) ** 0.5:.3e}"
 
 
