@@ -40,7 +40,10 @@ scaled_dot_product_attention for the attention): a yardstick for the hand-writte
 those routines is on the engine's path.
 `designs`: the Fedolorn decoder (gated attention with a chunked mask, squared-ReLU or routed-expert
 feed-forward) beside the Qwen2 decoder at equal sizes (`DESIGN_POINTS`): decode steps of the engine at
-`--batch` and one prompt step, for each; `--design-points` picks some of them.
+`--batch` and one prompt step, for each; `--design-points` picks some of them.  The points named
+`hybrid-*` (`BUBITAR_POINTS`; not among the default points) run the Bubitar decoder (retention layers and
+latent-attention layers in turn, sandwich norms, clamped gated feed-forward, a token input per layer) beside
+the Qwen2 decoder of the same width, heads, head size, feed-forward width, layers and vocabulary.
 `reference`: the reference's own published measurements, run here at their parameters with the
 0.5B shape (random weights and token ids of the published lengths; its figures are of an RTX 3060
 laptop GPU in float16 and stand beside for scale): the burst of 8 short requests under continuous and
@@ -100,7 +103,7 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
     p.add_argument("--seed", type=int, default=0)
     p.add_argument("--workload", default="decode", choices=("decode", "burst", "chunked", "library", "reference", "designs"))
-    p.add_argument("--design-only", default="", choices=("", "fedolorn", "qwen2"), help="run one of the two designs of the `designs` workload (for profiles)")
+    p.add_argument("--design-only", default="", choices=("", "fedolorn", "qwen2", "bubitar"), help="run one of the two designs of the `designs` workload (for profiles)")
     p.add_argument("--design-points", default="", help="names of the `designs` workload's points to run, comma separated (default: all)")
     p.add_argument("--no-large", action="store_true", help="leave out the 7B and 32B points of the default run")
     p.add_argument("--samples", action="store_true", help="print every raw sample, not only their summary")
@@ -781,9 +784,32 @@ class Bench:
                 + config.num_hidden_layers * config.num_attention_heads * 4 * d * tokens * (tokens + 1) // 2
                 + 2 * config.vocab_size * config.hidden_size
             )
+        width, flops = config.width, 2 * config.vocab * config.width
+        if hasattr(config, "token_side_dim"):
+            # retention: four input products, the state update and read (2 x dim x vdim a head and token, as the
+            # recurrence counts them), the output product; latent attention as the kernels run it: input
+            # product, the query through Wuk^T, scores and values over rows of kv_rank + rot_dim and kv_rank,
+            # the attended latent through Wuv, the output product; a gated feed-forward of three matrices;
+            # the token input's two small products
+            for layer in config.layers:
+                a, m = layer.mixer, layer.mlp
+                if a.kind == "retention":
+                    per_token = width * (2 * a.heads * a.dim + 2 * a.heads * a.vdim) + a.heads * a.vdim * width
+                    per_token += 2 * a.heads * a.dim * a.vdim
+                    pairs = 0
+                else:
+                    rows = a.heads * (a.dim + a.rot_dim) + a.heads + (0 if a.kv_from is not None else a.kv_rank + a.rot_dim)
+                    per_token = width * rows + a.heads * a.kv_rank * (a.dim + a.vdim) + a.heads * a.vdim * width
+                    pairs = tokens * (tokens + 1) // 2
+                if m is not None:
+                    per_token += 3 * width * m.ff
+                per_token += 2 * width * config.token_side_dim
+                flops += 2 * tokens * per_token
+                if pairs:
+                    flops += 2 * a.heads * (2 * a.kv_rank + a.rot_dim) * pairs
+            return flops
         # a configuration that lists its layers (attention with a gate and a chunked mask; dense or routed
         # feed-forward, of which a token uses `top` experts and the router)
-        width, flops = config.width, 2 * config.vocab * config.width
         for layer in config.layers:
             a, m = layer.mixer, layer.mlp
             per_token = width * (a.heads * a.dim + a.kv_heads * (a.dim + a.vdim) + 2 * a.heads * a.vdim)
@@ -845,7 +871,50 @@ DESIGN_POINTS = {
 DESIGN_VOCAB = 32768
 
 
+# The Bubitar decoder beside the Qwen2 decoder: the same width, query heads, head size, feed-forward width (both
+# feed-forwards have three matrices), layers and vocabulary.  Layers alternate retention (heads of dim x dim)
+# and latent attention (dim unrotated + 64 rotated query dimensions, a latent of 192: the cached row of 256 is
+# the widest the attention kernels take); every second latent layer reads the cache of the one before it.
+BUBITAR_POINTS = {
+    # name: (width, heads, kv heads of the Qwen2 twin, head size, feed-forward width, layers run, token side dim)
+    "hybrid-0.5b": (896, 14, 2, 64, 4864, 12, 64),
+    "hybrid-7b": (3584, 28, 4, 128, 18944, 4, 128),
+}
+
+
+def bubitar_configs(name: str) -> dict:
+    width, heads, kv_heads, dim, inter, layers, side = BUBITAR_POINTS[name]
+    rot = {"base": 1000000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    listed, owner = [], None
+    for i in range(layers):
+        if i % 2 == 0:
+            mixer = {"heads": heads, "dim": dim, "vdim": dim, "rot": {"base": 1000000.0, "dims": dim},
+                     "decay": [1.0 - 2.0 ** (-5 - 5 * h / max(1, heads - 1)) for h in range(heads)]}
+            kind = "retention"
+        else:
+            mixer = {"heads": heads, "dim": dim, "rot_dim": 64, "vdim": dim, "kv_rank": 192, "scale": (dim + 64) ** -0.5, "rot": rot}
+            if owner is not None:
+                mixer["kv_from"], owner = owner, None
+            else:
+                owner = i
+            kind = "latent_attention"
+        listed.append({"type": kind, "mixer": mixer, "mlp": {"kind": "dense", "ff": inter, "limit": 7.0}})
+    bubitar = {
+        "architecture": "Bubitar", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-5},
+        "token_side": {"dim": side}, "layers": listed,
+    }
+    qwen2 = {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "vocab_size": DESIGN_VOCAB, "hidden_size": width,
+        "intermediate_size": inter, "num_hidden_layers": layers, "num_attention_heads": heads,
+        "num_key_value_heads": kv_heads, "head_dim": dim, "max_position_embeddings": 32768, "rms_norm_eps": 1e-5,
+        "rope_theta": 1000000.0, "hidden_act": "silu", "tie_word_embeddings": True,
+    }
+    return {"bubitar": bubitar, "qwen2": qwen2}
+
+
 def design_configs(name: str) -> dict:
+    if name in BUBITAR_POINTS:
+        return bubitar_configs(name)
     width, heads, kv_heads, dim, inter, layers, mlp = DESIGN_POINTS[name]
     fedolorn = {
         "architecture": "Fedolorn", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-5},
@@ -890,8 +959,9 @@ def design_comparison(args) -> dict:
             bench.close()
             print(f"# {name} {design}: {point[design]}", file=sys.stderr, flush=True)
         if len(point) == 2:
-            point["decode_ratio"] = round(point["fedolorn"]["decode_tokens_per_s"] / point["qwen2"]["decode_tokens_per_s"], 3)
-            point["prefill_ratio"] = round(point["fedolorn"]["prefill_tokens_per_s"] / point["qwen2"]["prefill_tokens_per_s"], 3)
+            other = next(d for d in point if d != "qwen2")
+            point["decode_ratio"] = round(point[other]["decode_tokens_per_s"] / point["qwen2"]["decode_tokens_per_s"], 3)
+            point["prefill_ratio"] = round(point[other]["prefill_tokens_per_s"] / point["qwen2"]["prefill_tokens_per_s"], 3)
         points[name] = point
     return {
         "metric": "decode and prefill tokens/s of two designs at equal sizes",

@@ -189,10 +189,12 @@ int mlr_heads_linear(const void* x, int64_t in_row, int in_stride, const void* w
                      hipStream_t stream);
 
 // Retention over every entry's tokens in order, from and to rows of the state banks (see mixers.hip).
+// chunked: 64 tokens at a time on the matrix cores in true 32-bit (for entries of many tokens) instead of
+// token by token.
 int mlr_retention_scan(const float* projected, int width, float* state, int state_rows, const int* read_rows,
                        const int* write_rows, const int* cu_q, const int* q_starts, const float* decay,
                        const float* cos, const float* sin, int rotary_dims, float key_scale, float* out, int entries,
-                       int heads, int dim, int vdim, hipStream_t stream);
+                       int heads, int dim, int vdim, int chunked, hipStream_t stream);
 
 // out[t, h, :] = retained[t, h, :] / rms(retained[t, h, :]) * silu(projected[t, gate_offset + h * vdim + :]).
 int mlr_retention_gate(const float* retained, const float* projected, int width, int gate_offset, void* out, int dtype,

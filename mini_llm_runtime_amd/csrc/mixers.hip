@@ -8,6 +8,8 @@
 
 namespace mlr {
 
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
 // ---- x += weight * y * rsqrt(mean(y^2) + eps), then what reads the stream next -----------------
 // y is one tensor (float32 or the engine's dtype) or `slices` float32 partial sums added in slice
 // order.  mode 1: out = next_weight * x * rsqrt(mean(x^2) + next_eps); mode 2: out = x rounded to the
@@ -300,6 +302,153 @@ __global__ __launch_bounds__(64) void retention_scan_kernel(
   }
 }
 
+// The same recurrence for entries of many tokens, a chunk of 64 tokens at a time, on the matrix
+// cores in true 32-bit (v_mfma_f32_16x16x4_f32: operands and sums are float32).  With S the state
+// before a chunk of n tokens (local index i, j), g the decay and A_ij = (q_i . k_j) g^(i-j) for j <= i:
+//     o_i = g^(i+1) S^T q_i + sum_j A_ij v_j,      S' = g^n S + sum_j g^(n-1-j) k_j v_j^T.
+// A workgroup of four wavefronts owns 16 value columns of one head of one entry and walks the
+// entry's chunks in order; wavefront w owns the query rows 16 w .. 16 w + 15 of a chunk (score
+// tiles up to the diagonal, both output products) and every fourth 16-row tile of the state.
+// LDS: the chunk's rotated q and scaled k [64][dp + 1] (dp = dim rounded up to 16, zero padded), its
+// values [64][16], the masked scores per wavefront [16][65], the state [dp][16] and the powers g^0..g^64.
+// Lane layouts of the product D[16x16] += A[16x4] B[4x16]: lane l holds A[l % 16][l / 16],
+// B[l / 16][l % 16] and D[4 (l / 16) + e][l % 16], e = 0..3.
+constexpr int kChunk = 64;
+
+__device__ __forceinline__ f32x4v mfma_f32(float a, float b, f32x4v c) {
+  return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+__global__ __launch_bounds__(256) void retention_chunk_kernel(
+    const float* __restrict__ p, int width, float* __restrict__ state, const int* __restrict__ read_rows,
+    const int* __restrict__ write_rows, const int* __restrict__ cu_q, const int* __restrict__ q_starts,
+    const float* __restrict__ decay, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rdims,
+    float key_scale, float* __restrict__ out, int heads, int dim, int vdim, int dp) {
+  extern __shared__ float chunk_lds[];
+  const int ld = dp + 1;
+  float* const Qs = chunk_lds;                      // [64][ld]
+  float* const Ks = Qs + kChunk * ld;               // [64][ld]
+  float* const Vs = Ks + kChunk * ld;               // [64][16]
+  float* const As = Vs + kChunk * 16;               // [4][16][65]
+  float* const Ss = As + 4 * 16 * (kChunk + 1);     // [dp][16]
+  float* const pw = Ss + dp * 16;                   // [65]
+  const int entry = blockIdx.x;
+  const int h = blockIdx.y;
+  const int v0 = blockIdx.z * 16;
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave;
+  const int w = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int r16 = lane % 16;
+  const int quad = lane / 16;
+  const int t_first = cu_q[entry];
+  const int t_end = cu_q[entry + 1];
+  const float gamma = decay[h];
+  const int half = rdims / 2;
+  const int64_t head_state = static_cast<int64_t>(dim) * vdim;
+  float* const As_w = As + w * 16 * (kChunk + 1);
+
+  if (tid <= kChunk) pw[tid] = powf(gamma, static_cast<float>(tid));  // g^0 = 1 also when g = 0
+  const bool carried = q_starts[entry] > 0;
+  const float* src = state + (static_cast<int64_t>(read_rows[entry]) * heads + h) * head_state;
+  for (int idx = tid; idx < dp * 16; idx += 256) {
+    const int d = idx / 16, c = idx % 16;
+    Ss[idx] = (carried && d < dim && v0 + c < vdim) ? src[static_cast<int64_t>(d) * vdim + v0 + c] : 0.f;
+  }
+
+  for (int tb = t_first; tb < t_end; tb += kChunk) {
+    const int n = min(kChunk, t_end - tb);
+    __syncthreads();  // the chunk before is done with; the state is whole
+    for (int idx = tid; idx < kChunk * dp; idx += 256) {
+      const int i = idx / dp, d = idx - i * dp;
+      float qv = 0.f, kv = 0.f;
+      if (i < n && d < dim) {
+        const int64_t t = tb + i;
+        const float* q = p + t * width + static_cast<int64_t>(h) * dim;
+        const float* k = q + static_cast<int64_t>(heads) * dim;
+        qv = q[d];
+        kv = k[d];
+        if (d < rdims && cos_t != nullptr) {
+          const int j = d < half ? d : d - half;
+          const float cv = cos_t[t * half + j], sv = sin_t[t * half + j];
+          const int partner = d < half ? d + half : d - half;
+          const float sign = d < half ? -1.f : 1.f;
+          qv = qv * cv + sign * q[partner] * sv;
+          kv = kv * cv + sign * k[partner] * sv;
+        }
+        kv *= key_scale;
+      }
+      Qs[i * ld + d] = qv;
+      Ks[i * ld + d] = kv;
+    }
+    for (int idx = tid; idx < kChunk * 16; idx += 256) {
+      const int i = idx / 16, c = idx % 16;
+      Vs[idx] = (i < n && v0 + c < vdim)
+                    ? p[static_cast<int64_t>(tb + i) * width + 2ll * heads * dim + static_cast<int64_t>(h) * vdim + v0 + c]
+                    : 0.f;
+    }
+    __syncthreads();
+
+    // scores of this wavefront's 16 queries against the key tiles up to the diagonal, and the
+    // queries against the state; both read the same query operand
+    f32x4v sc[4], inter = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt) sc[jt] = f32x4v{0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < dp / 4; ++s) {
+      const int d = 4 * s + quad;
+      const float a = Qs[(16 * w + r16) * ld + d];
+      inter = mfma_f32(a, Ss[d * 16 + r16], inter);
+#pragma unroll
+      for (int jt = 0; jt < 4; ++jt)
+        if (jt <= w) sc[jt] = mfma_f32(a, Ks[(16 * jt + r16) * ld + d], sc[jt]);
+    }
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt) {
+      if (jt > w) continue;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int i = 16 * w + 4 * quad + e;  // query, key: local indices of the chunk
+        const int j = 16 * jt + r16;
+        As_w[(4 * quad + e) * (kChunk + 1) + j] = j <= i ? sc[jt][e] * pw[i - j] : 0.f;
+      }
+    }
+    __syncthreads();  // (a wavefront reads what its other lanes wrote)
+    f32x4v o = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < 4 * (w + 1); ++s) {
+      const int j = 4 * s + quad;
+      o = mfma_f32(As_w[r16 * (kChunk + 1) + j], Vs[j * 16 + r16], o);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int i = 16 * w + 4 * quad + e;
+      if (i < n && v0 + r16 < vdim)
+        out[static_cast<int64_t>(tb + i) * heads * vdim + static_cast<int64_t>(h) * vdim + v0 + r16] =
+            o[e] + pw[i + 1] * inter[e];
+    }
+    __syncthreads();  // every wavefront has read the state
+
+    // the state behind the chunk: rows of tile dt, for every fourth tile
+    for (int dt = w; dt < dp / 16; dt += 4) {
+      f32x4v up = {0.f, 0.f, 0.f, 0.f};
+      for (int s = 0; s < kChunk / 4; ++s) {
+        const int j = 4 * s + quad;
+        const float kj = j < n ? Ks[j * ld + 16 * dt + r16] * pw[n - 1 - j] : 0.f;
+        up = mfma_f32(kj, Vs[j * 16 + r16], up);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int d = 16 * dt + 4 * quad + e;
+        Ss[d * 16 + r16] = pw[n] * Ss[d * 16 + r16] + up[e];
+      }
+    }
+  }
+  __syncthreads();
+  float* dst = state + (static_cast<int64_t>(write_rows[entry]) * heads + h) * head_state;
+  for (int idx = tid; idx < dp * 16; idx += 256) {
+    const int d = idx / 16, c = idx % 16;
+    if (d < dim && v0 + c < vdim) dst[static_cast<int64_t>(d) * vdim + v0 + c] = Ss[idx];
+  }
+}
+
 // out[t, h, :] = o / sqrt(mean(o^2) + eps) * silu(z), o = retained[t, h, :] (float32), z = the gate sums at
 // column gate_offset + h * vdim of p [tokens, width] (float32).  One wavefront per (token, head).
 template <typename T>
@@ -425,7 +574,7 @@ int mlr_heads_linear(const void* x, int64_t in_row, int in_stride, const void* w
 int mlr_retention_scan(const float* projected, int width, float* state, int state_rows, const int* read_rows,
                        const int* write_rows, const int* cu_q, const int* q_starts, const float* decay,
                        const float* cos, const float* sin, int rotary_dims, float key_scale, float* out, int entries,
-                       int heads, int dim, int vdim, hipStream_t stream) {
+                       int heads, int dim, int vdim, int chunked, hipStream_t stream) {
   MLR_REQUIRE(projected && state && read_rows && write_rows && cu_q && q_starts && decay && out, "null pointer");
   MLR_REQUIRE(entries > 0 && heads > 0 && dim > 0 && vdim > 0 && state_rows > 0, "sizes must be > 0");
   MLR_REQUIRE(dim <= 256, "a head's state has up to 256 rows");
@@ -434,6 +583,24 @@ int mlr_retention_scan(const float* projected, int width, float* state, int stat
   MLR_REQUIRE(rotary_dims == 0 || (cos && sin), "a rotation needs cos and sin tables");
   dim3 grid(entries, heads, (vdim + 15) / 16);
   MLR_REQUIRE(grid.y < 65536u && grid.z < 65536u, "too many heads or columns for one launch");
+  if (chunked) {
+    const int dp = (dim + 15) / 16 * 16;
+    const size_t lds = (2 * kChunk * (dp + 1) + kChunk * 16 + 4 * 16 * (kChunk + 1) + dp * 16 + kChunk + 1) * sizeof(float);
+    static size_t configured = 0;
+    if (lds > 48 * 1024 && lds > configured) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(retention_chunk_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) {
+        set_error(std::string("mlr_retention_scan: cannot raise the LDS limit: ") + hipGetErrorString(e));
+        return -1;
+      }
+      configured = 160 * 1024;
+    }
+    retention_chunk_kernel<<<grid, 256, lds, stream>>>(projected, width, state, read_rows, write_rows, cu_q, q_starts,
+                                                       decay, cos, sin, rotary_dims, key_scale, out, heads, dim, vdim, dp);
+    MLR_LAUNCH_CHECK();
+    return 0;
+  }
 #define MLR_SCAN(dpl)                                                                                              \
   retention_scan_kernel<dpl><<<grid, 64, 0, stream>>>(projected, width, state, read_rows, write_rows, cu_q, q_starts, \
                                                       decay, cos, sin, rotary_dims, key_scale, out, heads, dim, vdim)

@@ -36,7 +36,7 @@ _SIGNATURES = {
         _I,
     ),
     "mlr_heads_linear": ([_VP, _I64, _I, _VP, _VP, _I64, _I, _VP, _I, _I, _I, _I, _I, _VP], _I),
-    "mlr_retention_scan": ([_VP, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _F, _VP, _I, _I, _I, _I, _VP], _I),
+    "mlr_retention_scan": ([_VP, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _F, _VP, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_retention_gate": ([_VP, _VP, _I, _I, _VP, _I, _I, _I, _I, _F, _VP], _I),
     "mlr_rmsnorm": ([_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _I, _F, _VP], _I),
     "mlr_add": ([_VP, _VP, _I, _I64, _VP], _I),
@@ -1088,6 +1088,8 @@ class HipOps:
         )
         return out
 
+    RETENTION_CHUNK_FROM = 4  # mean tokens an entry from which retention runs in chunks
+
     def retention_scan(
         self,
         projected: torch.Tensor,
@@ -1102,15 +1104,20 @@ class HipOps:
         decay: torch.Tensor,
         key_scale: float,
         rotation: Optional[tuple[torch.Tensor, torch.Tensor, int]],
+        chunked: Optional[bool] = None,
     ) -> torch.Tensor:
         """Retention of the step's tokens, every entry's in order: S = decay_h S + k v^T, o = S^T q per head,
         from the state in row read_rows[entry] of `state` [rows, heads, head_dim, value_dim] (zeros where the
         entry starts its request) to row write_rows[entry].  `projected` (float32 [T, >= 2 * heads * head_dim +
         heads * value_dim]) holds q, k and v; q and k are rotated and k scaled by `key_scale` here, in 32-bit.
-        Returns o, float32 [T, heads * value_dim]."""
+        Returns o, float32 [T, heads * value_dim].  Steps of single tokens (and of a few) run the recurrence
+        token by token with the state in registers; steps with longer entries run it 64 tokens at a time
+        on the matrix cores, in true 32-bit both ways (`chunked` forces one of them)."""
         self._check(projected, "projected input", torch.float32, (None, None))
         tokens, width = projected.shape
         entries = ctx.num_entries
+        if chunked is None:
+            chunked = tokens > self.RETENTION_CHUNK_FROM * entries  # more than a few tokens an entry
         self._check(state, "retention state", torch.float32, (None, heads, head_dim, value_dim))
         self._check(read_rows, "state rows to read", torch.int32, (entries,))
         self._check(write_rows, "state rows to write", torch.int32, (entries,))
@@ -1128,7 +1135,7 @@ class HipOps:
             "mlr_retention_scan", self._ptr(projected), width, self._ptr(state), state.shape[0], self._ptr(read_rows),
             self._ptr(write_rows), self._ptr(ctx.cu_q), self._ptr(ctx.q_starts), self._ptr(decay), self._ptr(cos),
             self._ptr(sin), int(rotary), float(key_scale), self._ptr(out), entries, heads, head_dim, value_dim,
-            self._stream(),
+            int(bool(chunked)), self._stream(),
         )
         return out
 

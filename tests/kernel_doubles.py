@@ -172,7 +172,8 @@ class TorchOps:
         return out
 
     def retention_scan(
-        self, projected, state, read_rows, write_rows, ctx, *, heads, head_dim, value_dim, decay, key_scale, rotation
+        self, projected, state, read_rows, write_rows, ctx, *, heads, head_dim, value_dim, decay, key_scale, rotation,
+        chunked=None,
     ):
         self._count("retention_scan")
         tokens = projected.shape[0]

@@ -387,16 +387,18 @@ def test_products_with_a_matrix_per_head(dtype, tokens, heads, n, k, stride):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("chunked", [False, True], ids=["by-token", "by-chunk"])
 @pytest.mark.parametrize("heads,dim,vdim,rdims", [(2, 16, 32, 8), (3, 20, 12, 20), (4, 64, 48, 64), (1, 128, 16, 0), (2, 200, 20, 100)])
-def test_retention_scan_and_its_state_rows(heads, dim, vdim, rdims):
-    """Three entries of unequal length, one of which goes on from a carried state; rows of other slots stay."""
+def test_retention_scan_and_its_state_rows(heads, dim, vdim, rdims, chunked):
+    """Three entries of unequal length (one token, less than a chunk of 64, two chunks and a bit), two of
+    which go on from a carried state; rows of other slots stay.  Token by token and in chunks."""
     ops = _ops("hip", torch.float32)
     g = torch.Generator().manual_seed(heads * dim + vdim)
-    lens, starts = [5, 1, 23], [0, 40, 7]
+    lens, starts = [5, 1, 150], [0, 40, 7]
     tokens = sum(lens)
     width = 2 * heads * dim + 2 * heads * vdim
     p = torch.randn(tokens, width, generator=g)
-    decay = torch.tensor([0.9, 0.99, 1.0, 0.5][:heads])
+    decay = torch.tensor([0.9, 0.99, 1.0, 0.0][:heads])  # also a head that forgets at once
     rot = {"base": 100.0, "dims": rdims}
     positions = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, lens)])
     bank = torch.randn(10, heads, dim, vdim, generator=g)  # stale values everywhere
@@ -407,11 +409,12 @@ def test_retention_scan_and_its_state_rows(heads, dim, vdim, rdims):
         angle = positions.double()[:, None] * f[None, :]
         rotation = (angle.cos().float().cuda(), angle.sin().float().cuda(), rdims)
     state = bank.clone().cuda()
-    cu = torch.tensor([0, 5, 6, 29], dtype=torch.int32)
+    cu = torch.tensor([0, 5, 6, 156], dtype=torch.int32)
     ctx = SimpleNamespace(num_entries=3, cu_q=cu.cuda(), q_starts=torch.tensor(starts, dtype=torch.int32).cuda())
     out = ops.retention_scan(
         p.cuda(), state, torch.tensor(read, dtype=torch.int32).cuda(), torch.tensor(write, dtype=torch.int32).cuda(), ctx,
         heads=heads, head_dim=dim, value_dim=vdim, decay=decay.cuda(), key_scale=dim**-0.5, rotation=rotation,
+        chunked=chunked,
     )
     qk = heads * dim
     for r in range(3):
