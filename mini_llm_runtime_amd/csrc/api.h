@@ -77,7 +77,7 @@ int mlr_qkv_finish(const float* partial, int slices, const float* cos, const flo
 // pairing) is multiplied into the activated sums: y = act(x w^T + bias) * multiply.
 int mlr_gemm_simple(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
                     int out_is_f32, int swiglu, int dtype, int m, int n, int k, const void* multiply,
-                    hipStream_t stream);
+                    float glu_limit, float glu_alpha, hipStream_t stream);
 
 // The same product in bfloat16 on the matrix cores (float32 accumulation).  Needs
 // k % 8 == 0 and 16-byte aligned x and w; any m and n.  With slices > 1 (a value
@@ -99,7 +99,7 @@ int mlr_gemm_bf16_kernel(int m, int n, int k, int slices);
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
                   int out_is_f32, int swiglu, int slices, int kernel, int m, int n, int k,
                   const float* row_sumsq, int sumsq_parts, float norm_eps, const void* multiply,
-                  hipStream_t stream);
+                  float glu_limit, float glu_alpha, hipStream_t stream);
 
 // A product that finishes the residual stream (gemm_stream.hip): y = a w^T (+ bias), a [m, k] and w
 // [n, k] bfloat16; then, every workgroup for its own columns of all rows, stream[m, n] (float32, in
@@ -190,11 +190,11 @@ int mlr_heads_linear(const void* x, int64_t in_row, int in_stride, const void* w
 
 // Retention over every entry's tokens in order, from and to rows of the state banks (see mixers.hip).
 // chunked: 64 tokens at a time on the matrix cores in true 32-bit (for entries of many tokens) instead of
-// token by token.
-int mlr_retention_scan(const float* projected, int width, float* state, int state_rows, const int* read_rows,
+// token by token; q and k of `projected` ([total_tokens, width]) are then rotated and scaled in place first.
+int mlr_retention_scan(float* projected, int width, float* state, int state_rows, const int* read_rows,
                        const int* write_rows, const int* cu_q, const int* q_starts, const float* decay,
                        const float* cos, const float* sin, int rotary_dims, float key_scale, float* out, int entries,
-                       int heads, int dim, int vdim, int chunked, hipStream_t stream);
+                       int heads, int dim, int vdim, int chunked, int total_tokens, hipStream_t stream);
 
 // out[t, h, :] = retained[t, h, :] / rms(retained[t, h, :]) * silu(projected[t, gate_offset + h * vdim + :]).
 int mlr_retention_gate(const float* retained, const float* projected, int width, int gate_offset, void* out, int dtype,

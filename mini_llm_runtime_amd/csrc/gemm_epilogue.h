@@ -27,13 +27,18 @@ struct GemmEpilogue {
   // [M, N] bfloat16, or null: the stored value is the (activated) sum times this, element by element
   // (a gate: sigmoid(x Wg^T) * other).  Not with kEpSwiglu, not with partial sums.
   const void* multiply = nullptr;
+  // kEpClampedGlu: rows woven as for kEpSwiglu (and the bias with them, which this pairing takes); stores
+  // g * sigmoid(glu_alpha * g) * (u + 1) with g = min(gate, glu_limit), u = clamp(up, -glu_limit, glu_limit).
+  float glu_limit = 0.f;
+  float glu_alpha = 0.f;
 };
 
 constexpr int kEpNone = 0;
 constexpr int kEpSwiglu = 1;
 constexpr int kEpRelu2 = 2;
 constexpr int kEpSigmoid = 3;
-constexpr int kEpGeluTanh = 4;  // 0.5 v (1 + tanh(sqrt(2 / pi) (v + 0.044715 v^3)))
+constexpr int kEpGeluTanh = 4;
+constexpr int kEpClampedGlu = 5;  // 0.5 v (1 + tanh(sqrt(2 / pi) (v + 0.044715 v^3)))
 
 // The scaling factors of rows m0 .. m0 + count - 1 into `scales` (LDS), by all wavefronts of the
 // workgroup (a whole number of them): wavefront w takes the rows w, w + waves, ..., its lanes the
@@ -117,11 +122,25 @@ template <bool ACTIVATIONS = true>
 __device__ __forceinline__ void store4(const GemmEpilogue& ep, int64_t m, int n, int N, float v0, float v1,
                                        float v2, float v3) {
   float v[4] = {v0, v1, v2, v3};
-  if (ep.swiglu == kEpSwiglu) {
+  bool paired = ep.swiglu == kEpSwiglu;
+  if constexpr (ACTIVATIONS) paired = paired || ep.swiglu == kEpClampedGlu;
+  if (paired) {
     // n..n+3 = gate 2j, gate 2j+1, up 2j, up 2j+1 with j = n / 4; N is a multiple of 4
     const int64_t at = m * (N / 2) + n / 2;
-    const float a = silu(v[0]) * v[2];
-    const float b = silu(v[1]) * v[3];
+    float a, b;
+    if (ep.swiglu == kEpSwiglu) {
+      a = silu(v[0]) * v[2];
+      b = silu(v[1]) * v[3];
+    } else {
+      if (ep.bias != nullptr) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] += load_as_f32(ep.bias, n + i, ep.bias_is_f32);
+      }
+      const float g0 = fminf(v[0], ep.glu_limit), g1 = fminf(v[1], ep.glu_limit);
+      const float u0 = fminf(fmaxf(v[2], -ep.glu_limit), ep.glu_limit), u1 = fminf(fmaxf(v[3], -ep.glu_limit), ep.glu_limit);
+      a = g0 / (1.0f + __expf(-ep.glu_alpha * g0)) * (u0 + 1.0f);
+      b = g1 / (1.0f + __expf(-ep.glu_alpha * g1)) * (u1 + 1.0f);
+    }
     if (ep.out_is_f32) {
       float* y = static_cast<float*>(ep.y) + at;
       y[0] = a;

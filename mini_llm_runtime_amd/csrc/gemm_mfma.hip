@@ -1132,11 +1132,15 @@ int mlr_gemm_bf16_kernel(int m, int n, int k, int slices) { return choose_kernel
 // over slices of k, the bias in slice 0, for the consumer to add up.
 // `swiglu` 2 and 3 are element-wise activations instead (squared ReLU, sigmoid; any n, after the
 // bias), and `multiply` (bfloat16 [m, n], or null) is multiplied into the activated sums.
+// `swiglu` 5: rows (and bias) woven as for 1, y [m, n / 2] = g * sigmoid(glu_alpha g) * (u + 1) with
+// g = min(gate, glu_limit), u = clamp(up, -glu_limit, glu_limit).
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y, int out_is_f32,
                   int swiglu, int slices, int kernel, int m, int n, int k, const float* row_sumsq, int sumsq_parts,
-                  float norm_eps, const void* multiply, hipStream_t stream) {
+                  float norm_eps, const void* multiply, float glu_limit, float glu_alpha, hipStream_t stream) {
   MLR_REQUIRE(x && w && y, "null pointer");
-  MLR_REQUIRE(swiglu >= kEpNone && swiglu <= kEpGeluTanh, "unknown epilogue");
+  MLR_REQUIRE(swiglu >= kEpNone && swiglu <= kEpClampedGlu, "unknown epilogue");
+  MLR_REQUIRE(swiglu != kEpClampedGlu || (n % 4 == 0 && multiply == nullptr && glu_limit > 0.f),
+              "the clamped gating needs n % 4 == 0, a limit > 0 and no multiplier");
   MLR_REQUIRE(multiply == nullptr || (swiglu != kEpSwiglu && slices == 1), "a multiplier goes with whole, unpaired sums");
   MLR_REQUIRE(slices == 1 || swiglu == kEpNone, "partial sums take no activation");
   MLR_REQUIRE(m > 0 && n > 0 && k > 0, "sizes must be > 0");
@@ -1149,7 +1153,7 @@ int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f3
               "x and w must be 16-byte aligned");
   MLR_REQUIRE(row_sumsq == nullptr || (sumsq_parts > 0 && sumsq_parts <= (1 << 16) && norm_eps >= 0.f),
               "sums of squares come with their number per row (1..65536) and an eps >= 0");
-  GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu, row_sumsq, sumsq_parts, norm_eps, multiply};
+  GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu, row_sumsq, sumsq_parts, norm_eps, multiply, glu_limit, glu_alpha};
   if (kernel == 0) kernel = choose_kernel(m, n, k, slices);
   // the 256 x 320 tile has no room for the activations and the multiplier in its epilogue
   if (kernel == 48 && (swiglu >= kEpRelu2 || multiply != nullptr)) kernel = 45;

@@ -19,7 +19,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                           const void* __restrict__ bias, int bias_is_f32,
                                                           void* __restrict__ y, int out_is_f32, int swiglu,
-                                                          const T* __restrict__ multiply, int M, int N, int K) {
+                                                          const T* __restrict__ multiply, int M, int N, int K,
+                                                          float glu_limit, float glu_alpha) {
   __shared__ float xs[kTK][kTM + 4];
   __shared__ float ws[kTK][kTN + 4];
   const int tid = threadIdx.x;
@@ -66,6 +67,28 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
   for (int i = 0; i < 4; ++i) {
     const int64_t gm = m0 + tm * 4 + i;
     if (gm >= M) continue;
+    if (swiglu == 5) {
+      // columns as for swiglu 1, the bias woven with them: g sigmoid(alpha g) (u + 1), both halves clamped
+      const int64_t gn = n0 + tn * 4;
+      if (gn >= N) continue;
+      const int64_t at = gm * (N / 2) + gn / 2;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        float g = acc[i][j], u = acc[i][j + 2];
+        if (bias != nullptr) {
+          g += load_as_f32(bias, gn + j, bias_is_f32);
+          u += load_as_f32(bias, gn + j + 2, bias_is_f32);
+        }
+        g = fminf(g, glu_limit);
+        u = fminf(fmaxf(u, -glu_limit), glu_limit);
+        const float v = g / (1.0f + expf(-glu_alpha * g)) * (u + 1.0f);
+        if (out_is_f32)
+          static_cast<float*>(y)[at + j] = v;
+        else
+          static_cast<T*>(y)[at + j] = from_f32<T>(v);
+      }
+      continue;
+    }
     if (swiglu == 1) {
       // columns n..n+3 = gate 2j, gate 2j+1, up 2j, up 2j+1 (rows of w interleaved in pairs);
       // qwen_model_runner.py:215-216: silu(gate) * up
@@ -112,25 +135,28 @@ using namespace mlr;
 
 extern "C" int mlr_gemm_simple(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
                                int out_is_f32, int swiglu, int dtype, int m, int n, int k, const void* multiply,
-                               hipStream_t stream) {
+                               float glu_limit, float glu_alpha, hipStream_t stream) {
   MLR_REQUIRE(x && w && y, "null pointer");
   MLR_REQUIRE(m > 0 && n > 0 && k > 0, "sizes must be > 0");
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
   MLR_REQUIRE(dtype == kBF16 || (out_is_f32 && (bias == nullptr || bias_is_f32)),
               "a float32 product has float32 bias and output");
-  MLR_REQUIRE(swiglu >= 0 && swiglu <= 4, "unknown epilogue");
+  MLR_REQUIRE(swiglu >= 0 && swiglu <= 5, "unknown epilogue");
   MLR_REQUIRE(swiglu != 1 || (n % 4 == 0 && bias == nullptr && multiply == nullptr),
               "swiglu needs n % 4 == 0, no bias and no multiplier");
+  MLR_REQUIRE(swiglu != 5 || (n % 4 == 0 && multiply == nullptr && glu_limit > 0.f),
+              "the clamped gating needs n % 4 == 0, a limit > 0 and no multiplier");
   dim3 grid((n + kTN - 1) / kTN, (m + kTM - 1) / kTM);
   MLR_REQUIRE(grid.y < 65536u, "too many rows for one launch");
   if (dtype == kF32)
     gemm_simple_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(x),
                                                         static_cast<const float*>(w), bias, bias_is_f32, y,
-                                                        out_is_f32, swiglu, static_cast<const float*>(multiply), m, n, k);
+                                                        out_is_f32, swiglu, static_cast<const float*>(multiply), m, n, k,
+                                                        glu_limit, glu_alpha);
   else
     gemm_simple_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w),
                                                        bias, bias_is_f32, y, out_is_f32, swiglu,
-                                                       static_cast<const bf16*>(multiply), m, n, k);
+                                                       static_cast<const bf16*>(multiply), m, n, k, glu_limit, glu_alpha);
   MLR_LAUNCH_CHECK();
   return 0;
 }

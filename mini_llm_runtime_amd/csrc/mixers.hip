@@ -57,6 +57,123 @@ __global__ __launch_bounds__(256) void add_normed_kernel(float* __restrict__ x, 
     orow[i] = from_f32<T>(load_as_f32(next_weight, i, next_is_f32) * (row_lds[i] * inv2));
 }
 
+// The same for rows whose width is a multiple of 4 and fits the registers of a workgroup: a thread keeps
+// VPT groups of 4 elements between the passes, and all loads of a pass (every slice of partial sums
+// included) are issued before the first is used: the kernel's time is the latency of its loads.
+template <typename T, int VPT, int THREADS>
+__global__ __launch_bounds__(THREADS) void add_normed_rows_kernel(
+    float* __restrict__ x, const void* __restrict__ y, int y_is_f32, int slices, int rows,
+    const void* __restrict__ weight, int weight_is_f32, float eps, const void* __restrict__ next_weight,
+    int next_is_f32, float next_eps, int mode, T* __restrict__ out, int hidden) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  const int quads = hidden / 4;
+  constexpr int kSliceBatch = 8;
+  f32x4v v[VPT], xv[VPT], wv[VPT], nv[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = min(static_cast<int>(threadIdx.x) + j * THREADS, quads - 1);
+    const int64_t at = row * hidden + 4 * i;
+    xv[j] = *reinterpret_cast<const f32x4v*>(x + at);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      wv[j][e] = load_as_f32(weight, 4 * i + e, weight_is_f32);
+      nv[j][e] = mode == 1 ? load_as_f32(next_weight, 4 * i + e, next_is_f32) : 0.f;
+    }
+    if (slices > 0) {
+      v[j] = f32x4v{0.f, 0.f, 0.f, 0.f};
+    } else if (y_is_f32) {
+      v[j] = *reinterpret_cast<const f32x4v*>(static_cast<const float*>(y) + at);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[j][e] = to_f32(static_cast<const T*>(y)[at + e]);
+    }
+  }
+  for (int s0 = 0; s0 < slices; s0 += kSliceBatch) {
+    f32x4v part[VPT][kSliceBatch];
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+      const int i = min(static_cast<int>(threadIdx.x) + j * THREADS, quads - 1);
+#pragma unroll
+      for (int u = 0; u < kSliceBatch; ++u) {
+        const int sl = min(s0 + u, slices - 1);
+        part[j][u] = *reinterpret_cast<const f32x4v*>(static_cast<const float*>(y) +
+                                                      (static_cast<int64_t>(sl) * rows + row) * hidden + 4 * i);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kSliceBatch; ++u) {
+      const bool live = s0 + u < slices;
+#pragma unroll
+      for (int j = 0; j < VPT; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[j][e] = live ? v[j][e] + part[j][u][e] : v[j][e];
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    if (static_cast<int>(threadIdx.x) + j * THREADS >= quads) v[j] = f32x4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss += v[j][e] * v[j][e];
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(hidden) + eps);
+  float ss2 = 0.f;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = threadIdx.x + j * THREADS;
+    if (i >= quads) {
+      xv[j] = f32x4v{0.f, 0.f, 0.f, 0.f};
+      continue;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      xv[j][e] += (v[j][e] * inv) * wv[j][e];
+      ss2 += xv[j][e] * xv[j][e];
+    }
+    *reinterpret_cast<f32x4v*>(x + row * hidden + 4 * i) = xv[j];
+  }
+  if (mode == 0) return;
+  float inv2 = 1.0f;
+  if (mode == 1) inv2 = 1.0f / sqrtf(block_sum(ss2, scratch) / static_cast<float>(hidden) + next_eps);
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = threadIdx.x + j * THREADS;
+    if (i >= quads) continue;
+    const int64_t at = row * hidden + 4 * i;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) out[at + e] = from_f32<T>(mode == 1 ? nv[j][e] * (xv[j][e] * inv2) : xv[j][e]);
+  }
+}
+
+template <typename T>
+static void launch_add_normed(float* x, const void* y, int y_is_f32, int slices, const void* weight, int weight_is_f32,
+                              float eps, const void* next_weight, int next_is_f32, float next_eps, int mode, void* out,
+                              int rows, int hidden, hipStream_t stream) {
+  T* o = static_cast<T*>(out);
+  const int quads = hidden / 4;
+#define MLR_ROWS(VPT, THREADS)                                                                                     \
+  add_normed_rows_kernel<T, VPT, THREADS><<<rows, THREADS, 0, stream>>>(x, y, y_is_f32, slices, rows, weight,     \
+                                                                        weight_is_f32, eps, next_weight, next_is_f32, \
+                                                                        next_eps, mode, o, hidden)
+  if (hidden % 4 != 0 || quads > 2048)
+    add_normed_kernel<T><<<rows, 256, static_cast<size_t>(hidden) * sizeof(float), stream>>>(
+        x, y, y_is_f32, slices, rows, weight, weight_is_f32, eps, next_weight, next_is_f32, next_eps, mode, o, hidden);
+  else if (rows <= 64 && quads > 512)
+    MLR_ROWS(2, 1024);
+  else if (rows <= 64 && quads > 256)
+    MLR_ROWS(1, 1024);
+  else if (quads <= 256)
+    MLR_ROWS(1, 256);
+  else if (quads <= 512)
+    MLR_ROWS(2, 256);
+  else if (quads <= 1024)
+    MLR_ROWS(4, 256);
+  else
+    MLR_ROWS(8, 256);
+#undef MLR_ROWS
+}
+
 // ---- g = min(gate, limit), u = clamp(up, -limit, limit): g * sigmoid(alpha g) * (u + 1) ---------
 // sums [rows, 2 * inter]: the gate sums, then the up sums.
 template <typename TI, typename T>
@@ -302,36 +419,70 @@ __global__ __launch_bounds__(64) void retention_scan_kernel(
   }
 }
 
+// q and k of `p` ([tokens, width] float32: q, then k, heads * dim each) rotated in place and k
+// scaled: what the chunked kernel below reads.  A thread owns a pair (d, d + rdims / 2) or an
+// unrotated dim.
+__global__ __launch_bounds__(256) void retention_rotate_kernel(float* __restrict__ p, int width,
+                                                               const float* __restrict__ cos_t,
+                                                               const float* __restrict__ sin_t, int rdims,
+                                                               float key_scale, int heads, int dim) {
+  const int64_t t = blockIdx.x;
+  const int half = rdims / 2;
+  float* q = p + t * width;
+  float* k = q + static_cast<int64_t>(heads) * dim;
+  for (int idx = threadIdx.x; idx < heads * dim; idx += 256) {
+    const int h = idx / dim;
+    const int d = idx - h * dim;
+    if (d >= rdims || cos_t == nullptr) {
+      k[idx] *= key_scale;
+    } else if (d < half) {
+      const float c = cos_t[t * half + d], sn = sin_t[t * half + d];
+      const float q0 = q[idx], q1 = q[idx + half], k0 = k[idx], k1 = k[idx + half];
+      q[idx] = q0 * c - q1 * sn;
+      q[idx + half] = q1 * c + q0 * sn;
+      k[idx] = (k0 * c - k1 * sn) * key_scale;
+      k[idx + half] = (k1 * c + k0 * sn) * key_scale;
+    }
+  }
+}
+
 // The same recurrence for entries of many tokens, a chunk of 64 tokens at a time, on the matrix
 // cores in true 32-bit (v_mfma_f32_16x16x4_f32: operands and sums are float32).  With S the state
 // before a chunk of n tokens (local index i, j), g the decay and A_ij = (q_i . k_j) g^(i-j) for j <= i:
 //     o_i = g^(i+1) S^T q_i + sum_j A_ij v_j,      S' = g^n S + sum_j g^(n-1-j) k_j v_j^T.
-// A workgroup of four wavefronts owns 16 value columns of one head of one entry and walks the
-// entry's chunks in order; wavefront w owns the query rows 16 w .. 16 w + 15 of a chunk (score
-// tiles up to the diagonal, both output products) and every fourth 16-row tile of the state.
-// LDS: the chunk's rotated q and scaled k [64][dp + 1] (dp = dim rounded up to 16, zero padded), its
-// values [64][16], the masked scores per wavefront [16][65], the state [dp][16] and the powers g^0..g^64.
+// q and k come rotated and scaled (retention_rotate_kernel).  A workgroup of four wavefronts owns 16
+// value columns of one head of one entry and walks the entry's chunks in order; wavefront w owns the
+// query rows 16 w .. 16 w + 15 of a chunk (score tiles up to the diagonal, both output products) and
+// every fourth 16-row tile of the state.  The next chunk's q, k and v are on their way from memory
+// (into registers) while a chunk is computed: the chain from chunk to chunk is arithmetic only.
+// LDS: the chunk's q and k [64][DP + 4] (DP: dim rounded up to 16, 32, 64 or 128, zero padded; rows
+// 4 words apart modulo 32 keep the operand reads of 16 rows x 4 columns off each other's banks), its
+// values [64][16], the masked scores per wavefront [16][68], the state [DP][16] and the powers g^0..g^64.
 // Lane layouts of the product D[16x16] += A[16x4] B[4x16]: lane l holds A[l % 16][l / 16],
 // B[l / 16][l % 16] and D[4 (l / 16) + e][l % 16], e = 0..3.
 constexpr int kChunk = 64;
+constexpr int kScoreLd = kChunk + 4;
 
 __device__ __forceinline__ f32x4v mfma_f32(float a, float b, f32x4v c) {
   return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
 }
 
+template <int DP>
 __global__ __launch_bounds__(256) void retention_chunk_kernel(
     const float* __restrict__ p, int width, float* __restrict__ state, const int* __restrict__ read_rows,
     const int* __restrict__ write_rows, const int* __restrict__ cu_q, const int* __restrict__ q_starts,
-    const float* __restrict__ decay, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rdims,
-    float key_scale, float* __restrict__ out, int heads, int dim, int vdim, int dp) {
+    const float* __restrict__ decay, float* __restrict__ out, int heads, int dim, int vdim) {
   extern __shared__ float chunk_lds[];
-  const int ld = dp + 1;
-  float* const Qs = chunk_lds;                      // [64][ld]
-  float* const Ks = Qs + kChunk * ld;               // [64][ld]
-  float* const Vs = Ks + kChunk * ld;               // [64][16]
-  float* const As = Vs + kChunk * 16;               // [4][16][65]
-  float* const Ss = As + 4 * 16 * (kChunk + 1);     // [dp][16]
-  float* const pw = Ss + dp * 16;                   // [65]
+  constexpr int LD = DP + 4;
+  constexpr int kPerRow = DP / 4;        // groups of 4 dims in a row
+  constexpr int kRowsAPass = 256 / kPerRow;
+  constexpr int kPasses = kChunk / kRowsAPass;
+  float* const Qs = chunk_lds;                    // [64][LD]
+  float* const Ks = Qs + kChunk * LD;             // [64][LD]
+  float* const Vs = Ks + kChunk * LD;             // [64][16]
+  float* const As = Vs + kChunk * 16;             // [4][16][kScoreLd]
+  float* const Ss = As + 4 * 16 * kScoreLd;       // [DP][16]
+  float* const pw = Ss + DP * 16;                 // [65]
   const int entry = blockIdx.x;
   const int h = blockIdx.y;
   const int v0 = blockIdx.z * 16;
@@ -343,14 +494,41 @@ __global__ __launch_bounds__(256) void retention_chunk_kernel(
   const int t_first = cu_q[entry];
   const int t_end = cu_q[entry + 1];
   const float gamma = decay[h];
-  const int half = rdims / 2;
   const int64_t head_state = static_cast<int64_t>(dim) * vdim;
-  float* const As_w = As + w * 16 * (kChunk + 1);
+  float* const As_w = As + w * 16 * kScoreLd;
+  const int64_t last = static_cast<int64_t>(t_end - 1);
+
+  // this thread's share of a chunk: 4 dims of `kPasses` rows of q and of k, 4 columns of one row of v;
+  // loads are unconditional (a row past the end reads the entry's last row, a dim past the head
+  // reads the head's last dim) and what does not exist is cleared when it goes to LDS
+  const int my_d = 4 * (tid % kPerRow);
+  const int my_row = tid / kPerRow;
+  const int v_row = tid / 4;
+  const int v_col = 4 * (tid % 4);
+  float qn[kPasses][4], kn[kPasses][4], vn[4];
+  auto fetch = [&](int tb) {
+#pragma unroll
+    for (int u = 0; u < kPasses; ++u) {
+      const int64_t t = min(static_cast<int64_t>(tb + u * kRowsAPass + my_row), last);
+      const float* q = p + t * width + static_cast<int64_t>(h) * dim;
+      const float* k = q + static_cast<int64_t>(heads) * dim;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int d = min(my_d + e, dim - 1);
+        qn[u][e] = q[d];
+        kn[u][e] = k[d];
+      }
+    }
+    const float* v = p + min(static_cast<int64_t>(tb + v_row), last) * width + 2ll * heads * dim + static_cast<int64_t>(h) * vdim;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) vn[e] = v[min(v0 + v_col + e, vdim - 1)];
+  };
+  fetch(t_first);
 
   if (tid <= kChunk) pw[tid] = powf(gamma, static_cast<float>(tid));  // g^0 = 1 also when g = 0
   const bool carried = q_starts[entry] > 0;
   const float* src = state + (static_cast<int64_t>(read_rows[entry]) * heads + h) * head_state;
-  for (int idx = tid; idx < dp * 16; idx += 256) {
+  for (int idx = tid; idx < DP * 16; idx += 256) {
     const int d = idx / 16, c = idx % 16;
     Ss[idx] = (carried && d < dim && v0 + c < vdim) ? src[static_cast<int64_t>(d) * vdim + v0 + c] : 0.f;
   }
@@ -358,48 +536,34 @@ __global__ __launch_bounds__(256) void retention_chunk_kernel(
   for (int tb = t_first; tb < t_end; tb += kChunk) {
     const int n = min(kChunk, t_end - tb);
     __syncthreads();  // the chunk before is done with; the state is whole
-    for (int idx = tid; idx < kChunk * dp; idx += 256) {
-      const int i = idx / dp, d = idx - i * dp;
-      float qv = 0.f, kv = 0.f;
-      if (i < n && d < dim) {
-        const int64_t t = tb + i;
-        const float* q = p + t * width + static_cast<int64_t>(h) * dim;
-        const float* k = q + static_cast<int64_t>(heads) * dim;
-        qv = q[d];
-        kv = k[d];
-        if (d < rdims && cos_t != nullptr) {
-          const int j = d < half ? d : d - half;
-          const float cv = cos_t[t * half + j], sv = sin_t[t * half + j];
-          const int partner = d < half ? d + half : d - half;
-          const float sign = d < half ? -1.f : 1.f;
-          qv = qv * cv + sign * q[partner] * sv;
-          kv = kv * cv + sign * k[partner] * sv;
-        }
-        kv *= key_scale;
+#pragma unroll
+    for (int u = 0; u < kPasses; ++u) {
+      const int i = u * kRowsAPass + my_row;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool there = i < n && my_d + e < dim;
+        Qs[i * LD + my_d + e] = there ? qn[u][e] : 0.f;
+        Ks[i * LD + my_d + e] = there ? kn[u][e] : 0.f;
       }
-      Qs[i * ld + d] = qv;
-      Ks[i * ld + d] = kv;
     }
-    for (int idx = tid; idx < kChunk * 16; idx += 256) {
-      const int i = idx / 16, c = idx % 16;
-      Vs[idx] = (i < n && v0 + c < vdim)
-                    ? p[static_cast<int64_t>(tb + i) * width + 2ll * heads * dim + static_cast<int64_t>(h) * vdim + v0 + c]
-                    : 0.f;
-    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) Vs[v_row * 16 + v_col + e] = (v_row < n && v0 + v_col + e < vdim) ? vn[e] : 0.f;
     __syncthreads();
+    if (tb + kChunk < t_end) fetch(tb + kChunk);  // on its way while this chunk is computed
 
     // scores of this wavefront's 16 queries against the key tiles up to the diagonal, and the
     // queries against the state; both read the same query operand
     f32x4v sc[4], inter = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int jt = 0; jt < 4; ++jt) sc[jt] = f32x4v{0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < dp / 4; ++s) {
+#pragma unroll 8
+    for (int s = 0; s < DP / 4; ++s) {
       const int d = 4 * s + quad;
-      const float a = Qs[(16 * w + r16) * ld + d];
+      const float a = Qs[(16 * w + r16) * LD + d];
       inter = mfma_f32(a, Ss[d * 16 + r16], inter);
 #pragma unroll
       for (int jt = 0; jt < 4; ++jt)
-        if (jt <= w) sc[jt] = mfma_f32(a, Ks[(16 * jt + r16) * ld + d], sc[jt]);
+        if (jt <= w) sc[jt] = mfma_f32(a, Ks[(16 * jt + r16) * LD + d], sc[jt]);
     }
 #pragma unroll
     for (int jt = 0; jt < 4; ++jt) {
@@ -408,14 +572,14 @@ __global__ __launch_bounds__(256) void retention_chunk_kernel(
       for (int e = 0; e < 4; ++e) {
         const int i = 16 * w + 4 * quad + e;  // query, key: local indices of the chunk
         const int j = 16 * jt + r16;
-        As_w[(4 * quad + e) * (kChunk + 1) + j] = j <= i ? sc[jt][e] * pw[i - j] : 0.f;
+        As_w[(4 * quad + e) * kScoreLd + j] = j <= i ? sc[jt][e] * pw[i - j] : 0.f;
       }
     }
     __syncthreads();  // (a wavefront reads what its other lanes wrote)
     f32x4v o = {0.f, 0.f, 0.f, 0.f};
     for (int s = 0; s < 4 * (w + 1); ++s) {
       const int j = 4 * s + quad;
-      o = mfma_f32(As_w[r16 * (kChunk + 1) + j], Vs[j * 16 + r16], o);
+      o = mfma_f32(As_w[r16 * kScoreLd + j], Vs[j * 16 + r16], o);
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -427,11 +591,12 @@ __global__ __launch_bounds__(256) void retention_chunk_kernel(
     __syncthreads();  // every wavefront has read the state
 
     // the state behind the chunk: rows of tile dt, for every fourth tile
-    for (int dt = w; dt < dp / 16; dt += 4) {
+    for (int dt = w; dt < DP / 16; dt += 4) {
       f32x4v up = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
       for (int s = 0; s < kChunk / 4; ++s) {
         const int j = 4 * s + quad;
-        const float kj = j < n ? Ks[j * ld + 16 * dt + r16] * pw[n - 1 - j] : 0.f;
+        const float kj = j < n ? Ks[j * LD + 16 * dt + r16] * pw[n - 1 - j] : 0.f;
         up = mfma_f32(kj, Vs[j * 16 + r16], up);
       }
 #pragma unroll
@@ -443,7 +608,7 @@ __global__ __launch_bounds__(256) void retention_chunk_kernel(
   }
   __syncthreads();
   float* dst = state + (static_cast<int64_t>(write_rows[entry]) * heads + h) * head_state;
-  for (int idx = tid; idx < dp * 16; idx += 256) {
+  for (int idx = tid; idx < DP * 16; idx += 256) {
     const int d = idx / 16, c = idx % 16;
     if (d < dim && v0 + c < vdim) dst[static_cast<int64_t>(d) * vdim + v0 + c] = Ss[idx];
   }
@@ -484,15 +649,12 @@ int mlr_add_normed(float* x, const void* y, int y_is_f32, int slices, const void
   MLR_REQUIRE(mode >= 0 && mode <= 2 && (mode == 0 || out) && (mode != 1 || next_weight), "bad mode or missing output");
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
   MLR_REQUIRE(dtype == kBF16 || y_is_f32, "a float32 engine has float32 activations");
-  const size_t lds = static_cast<size_t>(hidden) * sizeof(float);
   if (dtype == kF32)
-    add_normed_kernel<float><<<rows, 256, lds, stream>>>(x, y, y_is_f32, slices, rows, weight, weight_is_f32, eps,
-                                                         next_weight, next_is_f32, next_eps, mode,
-                                                         static_cast<float*>(out), hidden);
+    launch_add_normed<float>(x, y, y_is_f32, slices, weight, weight_is_f32, eps, next_weight, next_is_f32, next_eps, mode,
+                             out, rows, hidden, stream);
   else
-    add_normed_kernel<bf16><<<rows, 256, lds, stream>>>(x, y, y_is_f32, slices, rows, weight, weight_is_f32, eps,
-                                                        next_weight, next_is_f32, next_eps, mode,
-                                                        static_cast<bf16*>(out), hidden);
+    launch_add_normed<bf16>(x, y, y_is_f32, slices, weight, weight_is_f32, eps, next_weight, next_is_f32, next_eps, mode,
+                            out, rows, hidden, stream);
   MLR_LAUNCH_CHECK();
   return 0;
 }
@@ -571,10 +733,10 @@ int mlr_heads_linear(const void* x, int64_t in_row, int in_stride, const void* w
   return 0;
 }
 
-int mlr_retention_scan(const float* projected, int width, float* state, int state_rows, const int* read_rows,
+int mlr_retention_scan(float* projected, int width, float* state, int state_rows, const int* read_rows,
                        const int* write_rows, const int* cu_q, const int* q_starts, const float* decay,
                        const float* cos, const float* sin, int rotary_dims, float key_scale, float* out, int entries,
-                       int heads, int dim, int vdim, int chunked, hipStream_t stream) {
+                       int heads, int dim, int vdim, int chunked, int total_tokens, hipStream_t stream) {
   MLR_REQUIRE(projected && state && read_rows && write_rows && cu_q && q_starts && decay && out, "null pointer");
   MLR_REQUIRE(entries > 0 && heads > 0 && dim > 0 && vdim > 0 && state_rows > 0, "sizes must be > 0");
   MLR_REQUIRE(dim <= 256, "a head's state has up to 256 rows");
@@ -583,21 +745,35 @@ int mlr_retention_scan(const float* projected, int width, float* state, int stat
   MLR_REQUIRE(rotary_dims == 0 || (cos && sin), "a rotation needs cos and sin tables");
   dim3 grid(entries, heads, (vdim + 15) / 16);
   MLR_REQUIRE(grid.y < 65536u && grid.z < 65536u, "too many heads or columns for one launch");
-  if (chunked) {
-    const int dp = (dim + 15) / 16 * 16;
-    const size_t lds = (2 * kChunk * (dp + 1) + kChunk * 16 + 4 * 16 * (kChunk + 1) + dp * 16 + kChunk + 1) * sizeof(float);
-    static size_t configured = 0;
-    if (lds > 48 * 1024 && lds > configured) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(retention_chunk_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (chunked && dim <= 128) {  // wider heads keep the state of the token-by-token kernel
+    const int dp = dim <= 16 ? 16 : (dim <= 32 ? 32 : (dim <= 64 ? 64 : 128));
+    const size_t lds = (2 * kChunk * (dp + 4) + kChunk * 16 + 4 * 16 * kScoreLd + dp * 16 + kChunk + 1) * sizeof(float);
+    static bool configured = false;
+    if (!configured) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(retention_chunk_kernel<128>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
       if (e != hipSuccess) {
         set_error(std::string("mlr_retention_scan: cannot raise the LDS limit: ") + hipGetErrorString(e));
         return -1;
       }
-      configured = 160 * 1024;
+      configured = true;
     }
-    retention_chunk_kernel<<<grid, 256, lds, stream>>>(projected, width, state, read_rows, write_rows, cu_q, q_starts,
-                                                       decay, cos, sin, rotary_dims, key_scale, out, heads, dim, vdim, dp);
+    MLR_REQUIRE(total_tokens > 0, "the chunked kernel needs the number of tokens");
+    retention_rotate_kernel<<<total_tokens, 256, 0, stream>>>(const_cast<float*>(projected), width, cos, sin, rotary_dims,
+                                                              key_scale, heads, dim);
+    MLR_LAUNCH_CHECK();
+#define MLR_CHUNK(DP)                                                                                              \
+  retention_chunk_kernel<DP><<<grid, 256, lds, stream>>>(projected, width, state, read_rows, write_rows, cu_q, q_starts, \
+                                                         decay, out, heads, dim, vdim)
+    if (dp == 16)
+      MLR_CHUNK(16);
+    else if (dp == 32)
+      MLR_CHUNK(32);
+    else if (dp == 64)
+      MLR_CHUNK(64);
+    else
+      MLR_CHUNK(128);
+#undef MLR_CHUNK
     MLR_LAUNCH_CHECK();
     return 0;
   }

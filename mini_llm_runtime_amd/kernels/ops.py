@@ -36,7 +36,7 @@ _SIGNATURES = {
         _I,
     ),
     "mlr_heads_linear": ([_VP, _I64, _I, _VP, _VP, _I64, _I, _VP, _I, _I, _I, _I, _I, _VP], _I),
-    "mlr_retention_scan": ([_VP, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _F, _VP, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_retention_scan": ([_VP, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _F, _VP, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_retention_gate": ([_VP, _VP, _I, _I, _VP, _I, _I, _I, _I, _F, _VP], _I),
     "mlr_rmsnorm": ([_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _I, _F, _VP], _I),
     "mlr_add": ([_VP, _VP, _I, _I64, _VP], _I),
@@ -46,8 +46,8 @@ _SIGNATURES = {
     "mlr_rope_table": ([_VP, _VP, _VP, _VP, _I, _I, _F, _VP], _I),
     "mlr_rope_kv_write": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_qkv_finish": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
-    "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP], _I),
-    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _I, _VP, _I, _F, _VP, _VP], _I),
+    "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP, _F, _F, _VP], _I),
+    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _I, _VP, _I, _F, _VP, _F, _F, _VP], _I),
     "mlr_moe_route": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _VP], _I),
     "mlr_moe_tile_rows": ([_I], _I),
     "mlr_moe_max_tiles": ([_I, _I, _I], _I),
@@ -93,7 +93,7 @@ _SIGNATURES = {
 }
 
 # what `linear` may do to its sums before it stores them (the entry points' `swiglu` argument)
-_EPILOGUES = {None: 0, "swiglu": 1, "relu2": 2, "sigmoid": 3, "gelu_tanh": 4}
+_EPILOGUES = {None: 0, "swiglu": 1, "relu2": 2, "sigmoid": 3, "gelu_tanh": 4, "clamped_glu": 5}
 
 from .plans import PAGED_ATTENTION, QUERY_TILE, WIDE_QUERY_TILE, attention_plan, query_tiles  # noqa: F401
 
@@ -474,8 +474,13 @@ class HipOps:
         for_stream: bool = False,
         activation: Optional[str] = None,
         multiply: Optional[torch.Tensor] = None,
+        clamped_glu: Optional[tuple[float, float]] = None,
     ) -> torch.Tensor:
         """x [M, K] times weight [N, K] transposed, plus bias [N]; F.linear semantics.
+
+        clamped_glu: (limit, alpha).  The rows of `weight` (and the bias with them) are woven as for `swiglu`
+        (gate 2j, gate 2j+1, up 2j, up 2j+1) and the result is g * sigmoid(alpha g) * (u + 1), [M, N / 2], with
+        g = min(gate, limit) and u = clamp(up, -limit, limit): the pairing's other gating, with a bias.
 
         activation: "relu2" (max(v, 0)^2) or "sigmoid", applied to the sums (after the bias) in the
         product's epilogue, in 32-bit, before the one rounding to the output's dtype.
@@ -499,11 +504,22 @@ class HipOps:
         """
         if kernel not in ("auto", "fma"):
             raise KernelError("kernel must be 'auto' or 'fma'")
-        if activation not in _EPILOGUES or activation == "swiglu":
+        if activation not in _EPILOGUES or activation in ("swiglu", "clamped_glu"):
             raise KernelError(f"unknown activation {activation!r}")
+        glu_limit = glu_alpha = 0.0
+        if clamped_glu is not None:
+            if swiglu or activation is not None or multiply is not None or partial_sums or for_stream or slices not in (None, 1):
+                raise KernelError("the clamped gating goes with whole sums and nothing else")
+            glu_limit, glu_alpha = float(clamped_glu[0]), float(clamped_glu[1])
+            if not glu_limit > 0:
+                raise KernelError("the clamped gating needs a limit > 0")
+            x = self.settle(x)  # no fused prologue knows this pairing
         if (activation is not None or multiply is not None) and (swiglu or partial_sums or for_stream or slices not in (None, 1)):
             raise KernelError("an activation or a multiplier goes with whole sums: no SwiGLU pairing, no slices of k")
         epilogue = 1 if swiglu else _EPILOGUES[activation]
+        if clamped_glu is not None:
+            epilogue = _EPILOGUES["clamped_glu"]
+            swiglu = True  # for the shape of the result; the bias check below is the pairing-without-bias one
         if for_stream:
             partial_sums = True
             m, k = x.shape
@@ -531,7 +547,7 @@ class HipOps:
         n = weight.shape[0]
         if bias is not None:
             self._check(bias, "linear bias", (torch.float32, self.dtype), (n,))
-        if swiglu and (n % 4 or bias is not None):
+        if swiglu and (n % 4 or (bias is not None and clamped_glu is None)):
             raise KernelError("a SwiGLU product needs a multiple of 4 rows and no bias")
         out_dtype = out_dtype or self.dtype
         if out_dtype not in (torch.float32, self.dtype):
@@ -554,13 +570,15 @@ class HipOps:
                 out_f32 = int(out_dtype == torch.float32)
             self._call(
                 "mlr_gemm_bf16", self._ptr(x), self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y), out_f32,
-                epilogue, slices, int(mfma_kernel), m, n, k, *scale, self._ptr(multiply), self._stream(),
+                epilogue, slices, int(mfma_kernel), m, n, k, *scale, self._ptr(multiply), glu_limit, glu_alpha,
+                self._stream(),
             )
             return y
         y = self._empty((m, n // 2 if swiglu else n), out_dtype)
         self._call(
             "mlr_gemm_simple", self._ptr(x), self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y),
-            int(out_dtype == torch.float32), epilogue, self.code, m, n, k, self._ptr(multiply), self._stream(),
+            int(out_dtype == torch.float32), epilogue, self.code, m, n, k, self._ptr(multiply), glu_limit, glu_alpha,
+            self._stream(),
         )
         return y
 
@@ -1109,7 +1127,8 @@ class HipOps:
         """Retention of the step's tokens, every entry's in order: S = decay_h S + k v^T, o = S^T q per head,
         from the state in row read_rows[entry] of `state` [rows, heads, head_dim, value_dim] (zeros where the
         entry starts its request) to row write_rows[entry].  `projected` (float32 [T, >= 2 * heads * head_dim +
-        heads * value_dim]) holds q, k and v; q and k are rotated and k scaled by `key_scale` here, in 32-bit.
+        heads * value_dim]) holds q, k and v; q and k are rotated and k scaled by `key_scale` here, in 32-bit
+        (the chunked way does that in place: `projected` is the caller's scratch).
         Returns o, float32 [T, heads * value_dim].  Steps of single tokens (and of a few) run the recurrence
         token by token with the state in registers; steps with longer entries run it 64 tokens at a time
         on the matrix cores, in true 32-bit both ways (`chunked` forces one of them)."""
@@ -1135,7 +1154,7 @@ class HipOps:
             "mlr_retention_scan", self._ptr(projected), width, self._ptr(state), state.shape[0], self._ptr(read_rows),
             self._ptr(write_rows), self._ptr(ctx.cu_q), self._ptr(ctx.q_starts), self._ptr(decay), self._ptr(cos),
             self._ptr(sin), int(rotary), float(key_scale), self._ptr(out), entries, heads, head_dim, value_dim,
-            int(bool(chunked)), self._stream(),
+            int(bool(chunked)), tokens, self._stream(),
         )
         return out
 

@@ -101,13 +101,17 @@ def bubitar_spec(config: BubitarConfig) -> ModelSpec:
             norms.update(post_mixer=norm, ff_out=norm)
             feed_forward = PartSpec("clamped_glu", {"hidden_size": width, "intermediate_size": f.ff, "limit": f.limit})
             ff = dst + "feed_forward."
+            # gate and up rows (and biases) woven in pairs: the product's epilogue then holds a gate sum
+            # beside its up sum (an odd size cannot be woven: gate rows, then up rows)
+            weave = dict(block=2, period=4) if f.ff % 2 == 0 else {}
+            up_at = 2 if weave else f.ff
             rules += [
                 WeightRule(src + "norm2", dst + "norm_post_mixer.weight"),
                 WeightRule(src + "norm2b", dst + "norm_ff_out.weight"),
-                WeightRule(src + "mlp.gate", ff + "gate_up_weight", 0, f.ff),
-                WeightRule(src + "mlp.up", ff + "gate_up_weight", f.ff, f.ff),
-                WeightRule(src + "mlp.gate.b", ff + "gate_up_bias", 0, f.ff),
-                WeightRule(src + "mlp.up.b", ff + "gate_up_bias", f.ff, f.ff),
+                WeightRule(src + "mlp.gate", ff + "gate_up_weight", 0, f.ff, **weave),
+                WeightRule(src + "mlp.up", ff + "gate_up_weight", up_at, f.ff, **weave),
+                WeightRule(src + "mlp.gate.b", ff + "gate_up_bias", 0, f.ff, **weave),
+                WeightRule(src + "mlp.up.b", ff + "gate_up_bias", up_at, f.ff, **weave),
                 WeightRule(src + "mlp.down", ff + "down_weight"),
                 WeightRule(src + "mlp.down.b", ff + "down_bias"),
             ]

@@ -52,7 +52,10 @@ class ClampedGLU(FeedForward):
         g = min(Wgate x + bgate, limit),  u = clamp(Wup x + bup, -limit, limit),
         y = Wdown (g * sigmoid(alpha * g) * (u + 1)) + bdown.
 
-    Gate and up are one product over the rows [Wgate ; Wup]; the gating reads its 32-bit sums.
+    Gate and up are one product over a matrix that holds the rows of Wgate and Wup woven in pairs (gate
+    0, gate 1, up 0, up 1, gate 2, ...; made by the weight rules, the biases alike), and the gating is that
+    product's epilogue, on its 32-bit sums.  An odd intermediate size cannot be woven in pairs (`woven` is
+    False): its rows are [Wgate ; Wup] and the gating is a kernel of its own behind the product.
     """
 
     replayable = True
@@ -64,6 +67,7 @@ class ClampedGLU(FeedForward):
         self.intermediate_size = int(intermediate_size)
         self.limit = float(limit)
         self.alpha = float(alpha)
+        self.woven = self.intermediate_size % 2 == 0
         self.gate_up_weight: Optional[torch.Tensor] = None
         self.gate_up_bias: Optional[torch.Tensor] = None
         self.down_weight: Optional[torch.Tensor] = None
@@ -79,8 +83,11 @@ class ClampedGLU(FeedForward):
 
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
         ops = ctx.ops
-        sums = ops.linear(h, self.gate_up_weight, self.gate_up_bias, out_dtype=torch.float32)
-        hidden = ops.glu_clamped(sums, self.limit, self.alpha)
+        if self.woven:
+            hidden = ops.linear(h, self.gate_up_weight, self.gate_up_bias, clamped_glu=(self.limit, self.alpha))
+        else:
+            sums = ops.linear(h, self.gate_up_weight, self.gate_up_bias, out_dtype=torch.float32)
+            hidden = ops.glu_clamped(sums, self.limit, self.alpha)
         return ops.linear(hidden, self.down_weight, self.down_bias, for_stream=True)
 
 

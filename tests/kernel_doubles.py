@@ -78,7 +78,7 @@ class TorchOps:
     # matrix products ---------------------------------------------------------------------
     def linear(
         self, x, weight, bias=None, out_dtype=None, kernel="auto", swiglu=False, partial_sums=False, for_stream=False,
-        activation=None, multiply=None,
+        activation=None, multiply=None, clamped_glu=None,
     ):
         self._count("linear")
         y = x.float() @ weight.float().t()
@@ -94,6 +94,12 @@ class TorchOps:
             raise ValueError(activation)
         if multiply is not None:
             y = y * multiply.float()
+        if clamped_glu is not None:  # rows woven like swiglu's, the bias with them
+            limit, alpha = clamped_glu
+            quads = y.view(y.shape[0], -1, 4)
+            gate = quads[..., :2].clamp(max=limit)
+            up = quads[..., 2:].clamp(-limit, limit)
+            y = (gate * torch.sigmoid(alpha * gate) * (up + 1.0)).reshape(y.shape[0], -1)
         if swiglu:  # rows of weight: gate 2j, gate 2j+1, up 2j, up 2j+1
             quads = y.view(y.shape[0], -1, 4)
             gate, up = quads[..., :2], quads[..., 2:]

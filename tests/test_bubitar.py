@@ -80,7 +80,7 @@ CONFIGS = {
     # of 12, an odd side dim, an odd vocabulary, retention heads of 20 x 12
     "B": _model(257, 72, 1e-5, 5, [
         (_retention(3, 20, 12, (0.95, 0.9, 0.999), _rot(777.0, 20)), _ff(52, 1.3)),
-        (_latent(3, 10, 6, 12, 20, 0.3, _rot(3000.0, 4)), _ff(44, 0.6)),
+        (_latent(3, 10, 6, 12, 20, 0.3, _rot(3000.0, 4)), _ff(45, 0.6)),
     ]),
     # matrix-core sizes: a cached row of 96 + 32 = 128, eight heads on it; retention heads of 64 x 32
     "C": _model(512, 128, 1e-5, 16, [
@@ -309,7 +309,7 @@ def _tolerance(dtype):
 
 
 @pytest.mark.parametrize("dtype", GPU_CASES)
-@pytest.mark.parametrize("rows,size,slices", [(1, 64, 0), (7, 100, 3), (300, 192, 0), (3, 2048, 2), (5, 72, 1)])
+@pytest.mark.parametrize("rows,size,slices", [(1, 64, 0), (7, 100, 3), (300, 192, 0), (3, 2048, 2), (5, 72, 1), (4, 70, 2), (2, 8196, 1), (8, 3584, 11), (70, 4096, 0)])
 def test_normed_addition(dtype, rows, size, slices):
     ops = _ops("hip", dtype)
     g = torch.Generator().manual_seed(rows + size)
@@ -348,6 +348,25 @@ def test_clamped_gating(dtype, rows, inner, limit):
     gate = torch.clamp(sums[:, :inner].double(), max=limit)
     up = torch.clamp(sums[:, inner:].double(), -limit, limit)
     assert float((sums[:, :inner] < -limit).float().mean()) > 0.02  # the gate has no lower clamp: such values must pass
+    torch.testing.assert_close(got.double().cpu(), gate * torch.sigmoid(1.702 * gate) * (up + 1.0), **_tolerance(dtype))
+
+
+@pytest.mark.parametrize("dtype", GPU_CASES)
+@pytest.mark.parametrize("m,inner,k,limit", [(1, 40, 64, 1.0), (5, 26, 72, 0.6), (33, 128, 100, 2.5), (300, 256, 128, 1.0), (64, 640, 256, 1.5), (2048, 320, 512, 0.9)])
+def test_clamped_gating_as_the_epilogue_of_its_product(dtype, m, inner, k, limit):
+    """Gate and up rows woven in pairs, the biases with them; every product kernel that a shape may choose."""
+    ops = _ops("hip", dtype)
+    g = torch.Generator().manual_seed(m + inner + k)
+    x = torch.randn(m, k, generator=g).to(dtype)
+    wg = (torch.randn(inner, k, generator=g) * 2.0 / math.sqrt(k)).to(dtype)
+    wu = (torch.randn(inner, k, generator=g) * 2.0 / math.sqrt(k)).to(dtype)
+    bg, bu = torch.randn(inner, generator=g) * 0.5, torch.randn(inner, generator=g) * 0.5
+    woven = torch.stack([wg.view(-1, 2, k), wu.view(-1, 2, k)], dim=1).reshape(2 * inner, k).contiguous()
+    bias = torch.stack([bg.view(-1, 2), bu.view(-1, 2)], dim=1).reshape(2 * inner).contiguous()
+    got = ops.linear(x.cuda(), woven.cuda(), bias.cuda(), clamped_glu=(limit, 1.702))
+    gate = torch.clamp(x.double() @ wg.double().T + bg.double(), max=limit)
+    up = torch.clamp(x.double() @ wu.double().T + bu.double(), -limit, limit)
+    assert got.shape == (m, inner) and got.dtype == dtype
     torch.testing.assert_close(got.double().cpu(), gate * torch.sigmoid(1.702 * gate) * (up + 1.0), **_tolerance(dtype))
 
 
