@@ -5,6 +5,7 @@
 // All arithmetic is float32; bfloat16 only exists in memory.
 #include "api.h"
 #include "common.h"
+#include "mfma.h"
 
 namespace mlr {
 
@@ -319,6 +320,53 @@ __global__ __launch_bounds__(256) void heads_linear_kernel(const T* __restrict__
     for (int j = 0; j < 4; ++j) {
       const int64_t gn = n0 + tn * 4 + j;
       if (gn < N) out[gm * out_row + static_cast<int64_t>(h) * out_stride + gn] = from_f32<T>(acc[i][j] * s);
+    }
+  }
+}
+
+// The same product in bfloat16 on the matrix cores: a wavefront owns 16 tokens x (16 NT) outputs of one
+// head and reads both operands straight from memory, 8 consecutive k a lane (the matrices are small:
+// what one wavefront reads again, another has left in L2).  The weights are the A operand, so a lane
+// ends up with 4 consecutive outputs of one token.  k is a multiple of 8; rows and head strides keep
+// every 8 k values 16-byte aligned.
+template <int NT>
+__global__ __launch_bounds__(64) void heads_linear_mfma_kernel(const bf16* __restrict__ x, int64_t in_row, int in_stride,
+                                                               const bf16* __restrict__ w, bf16* __restrict__ out,
+                                                               int64_t out_row, int out_stride,
+                                                               const float* __restrict__ row_scale, int heads, int M,
+                                                               int N, int K) {
+  const int lane = threadIdx.x;
+  const int r16 = lane % 16;
+  const int quad = lane / 16;
+  const int h = blockIdx.z;
+  const int m0 = blockIdx.y * 16;
+  const int n0 = blockIdx.x * 16 * NT;
+  const int t = min(m0 + r16, M - 1);  // rows past the end read the last row; their results are dropped
+  const bf16* xrow = x + static_cast<int64_t>(t) * in_row + static_cast<int64_t>(h) * in_stride;
+  const bf16* wh = w + static_cast<int64_t>(h) * N * K;
+  f32x4_t acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const int k = k0 + quad * 8;
+    const bool inside = k < K;
+    const bf16x8_t b = inside ? load_bf16x8(xrow + k) : zero_bf16x8();
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int n = min(n0 + 16 * j + r16, N - 1);
+      const bf16x8_t a = inside ? load_bf16x8(wh + static_cast<int64_t>(n) * K + k) : zero_bf16x8();
+      acc[j] = mfma_16x16x32(a, b, acc[j]);
+    }
+  }
+  if (m0 + r16 >= M) return;
+  const float scale = row_scale ? row_scale[static_cast<int64_t>(m0 + r16) * heads + h] : 1.0f;
+  bf16* orow = out + static_cast<int64_t>(m0 + r16) * out_row + static_cast<int64_t>(h) * out_stride;
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int n = n0 + 16 * j + 4 * quad + e;
+      if (n < N) orow[n] = f32_to_bf16(acc[j][e] * scale);
     }
   }
 }
@@ -719,6 +767,21 @@ int mlr_heads_linear(const void* x, int64_t in_row, int in_stride, const void* w
   MLR_REQUIRE(in_stride >= k && in_row >= static_cast<int64_t>(heads) * in_stride, "the input rows do not hold every head's k values");
   MLR_REQUIRE(out_stride >= n && out_row >= static_cast<int64_t>(heads) * out_stride, "the output rows do not hold every head's n values");
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  MLR_REQUIRE(heads < 65536 && (tokens + 15) / 16 < 65536, "too many rows or heads for one launch");
+  if (dtype == kBF16 && k % 8 == 0 && in_stride % 8 == 0 && in_row % 8 == 0 &&
+      reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0) {
+    // few tokens: a wavefront per 16 outputs, so that many compute units share the weights' bytes
+    if (tokens <= 64)
+      heads_linear_mfma_kernel<1><<<dim3((n + 15) / 16, (tokens + 15) / 16, heads), 64, 0, stream>>>(
+          static_cast<const bf16*>(x), in_row, in_stride, static_cast<const bf16*>(w), static_cast<bf16*>(out), out_row,
+          out_stride, row_scale, heads, tokens, n, k);
+    else
+      heads_linear_mfma_kernel<4><<<dim3((n + 63) / 64, (tokens + 15) / 16, heads), 64, 0, stream>>>(
+          static_cast<const bf16*>(x), in_row, in_stride, static_cast<const bf16*>(w), static_cast<bf16*>(out), out_row,
+          out_stride, row_scale, heads, tokens, n, k);
+    MLR_LAUNCH_CHECK();
+    return 0;
+  }
   dim3 grid((n + 63) / 64, (tokens + 63) / 64, heads);
   MLR_REQUIRE(grid.y < 65536u && grid.z < 65536u, "too many rows or heads for one launch");
   if (dtype == kF32)

@@ -387,7 +387,7 @@ def test_gelu_product_with_gathered_rows(dtype, m, n, k):
 
 
 @pytest.mark.parametrize("dtype", GPU_CASES)
-@pytest.mark.parametrize("tokens,heads,n,k,stride", [(1, 2, 40, 16, 16), (70, 3, 20, 10, 10), (130, 8, 32, 96, 128), (9, 4, 100, 64, 80)])
+@pytest.mark.parametrize("tokens,heads,n,k,stride", [(1, 2, 40, 16, 16), (70, 3, 20, 10, 10), (130, 8, 32, 96, 128), (9, 4, 100, 64, 80), (5, 2, 24, 40, 48), (300, 3, 70, 72, 72)])
 def test_products_with_a_matrix_per_head(dtype, tokens, heads, n, k, stride):
     ops = _ops("hip", dtype)
     g = torch.Generator().manual_seed(tokens + heads)
