@@ -190,11 +190,14 @@ int mlr_heads_linear(const void* x, int64_t in_row, int in_stride, const void* w
 
 // Retention over every entry's tokens in order, from and to rows of the state banks (see mixers.hip).
 // chunked: 64 tokens at a time on the matrix cores in true 32-bit (for entries of many tokens) instead of
-// token by token; q and k of `projected` ([total_tokens, width]) are then rotated and scaled in place first.
+// token by token; q and k of `projected` ([total_tokens, width]) are then rotated and scaled in place first,
+// and `scratch` holds mlr_retention_scratch floats (what every chunk adds to the state).
+int64_t mlr_retention_scratch(int total_tokens, int entries, int heads, int dim, int vdim);
 int mlr_retention_scan(float* projected, int width, float* state, int state_rows, const int* read_rows,
                        const int* write_rows, const int* cu_q, const int* q_starts, const float* decay,
                        const float* cos, const float* sin, int rotary_dims, float key_scale, float* out, int entries,
-                       int heads, int dim, int vdim, int chunked, int total_tokens, hipStream_t stream);
+                       int heads, int dim, int vdim, int chunked, int total_tokens, float* scratch, int64_t scratch_floats,
+                       hipStream_t stream);
 
 // out[t, h, :] = retained[t, h, :] / rms(retained[t, h, :]) * silu(projected[t, gate_offset + h * vdim + :]).
 int mlr_retention_gate(const float* retained, const float* projected, int width, int gate_offset, void* out, int dtype,

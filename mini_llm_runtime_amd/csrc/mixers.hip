@@ -497,15 +497,18 @@ __global__ __launch_bounds__(256) void retention_rotate_kernel(float* __restrict
 // The same recurrence for entries of many tokens, a chunk of 64 tokens at a time, on the matrix
 // cores in true 32-bit (v_mfma_f32_16x16x4_f32: operands and sums are float32).  With S the state
 // before a chunk of n tokens (local index i, j), g the decay and A_ij = (q_i . k_j) g^(i-j) for j <= i:
-//     o_i = g^(i+1) S^T q_i + sum_j A_ij v_j,      S' = g^n S + sum_j g^(n-1-j) k_j v_j^T.
-// q and k come rotated and scaled (retention_rotate_kernel).  A workgroup of four wavefronts owns 16
-// value columns of one head of one entry and walks the entry's chunks in order; wavefront w owns the
-// query rows 16 w .. 16 w + 15 of a chunk (score tiles up to the diagonal, both output products) and
-// every fourth 16-row tile of the state.  The next chunk's q, k and v are on their way from memory
-// (into registers) while a chunk is computed: the chain from chunk to chunk is arithmetic only.
-// LDS: the chunk's q and k [64][DP + 4] (DP: dim rounded up to 16, 32, 64 or 128, zero padded; rows
-// 4 words apart modulo 32 keep the operand reads of 16 rows x 4 columns off each other's banks), its
-// values [64][16], the masked scores per wavefront [16][68], the state [DP][16] and the powers g^0..g^64.
+//     o_i = g^(i+1) S^T q_i + sum_j A_ij v_j,      S' = g^n S + U,   U = sum_j g^(n-1-j) k_j v_j^T.
+// q and k come rotated and scaled (retention_rotate_kernel).  Only S links the chunks, so the work is
+// cut in two.  retention_local_kernel: a workgroup per (chunk, head, 16 value columns), all chunks of
+// all entries at once, makes the chunk's own part of o (the sum over j) and its U.
+// retention_carry_kernel: a workgroup per (entry, head, 16 value columns) walks the entry's chunks in
+// order, adds g^(i+1) S^T q_i to o and moves S on by U: one small product and two barriers a chunk, its
+// operands asked for a chunk ahead.
+// Wavefront w of four owns the query rows 16 w .. 16 w + 15 of a chunk and every fourth 16-row tile of
+// the state.  LDS of the first kernel: the chunk's q and k [64][DP + 4] (DP: dim rounded up to 16, 32,
+// 64 or 128, zero padded; rows 4 words apart modulo 32 keep the operand reads of 16 rows x 4 columns
+// off each other's banks), its values [64][16], the masked scores per wavefront [16][68], the powers
+// g^0..g^64; of the second: the state [DP][16] and the powers.
 // Lane layouts of the product D[16x16] += A[16x4] B[4x16]: lane l holds A[l % 16][l / 16],
 // B[l / 16][l % 16] and D[4 (l / 16) + e][l % 16], e = 0..3.
 constexpr int kChunk = 64;
@@ -515,22 +518,140 @@ __device__ __forceinline__ f32x4v mfma_f32(float a, float b, f32x4v c) {
   return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
 }
 
+// Chunks are numbered through the entries in order, an entry of n tokens having ceil(n / 64).
+__device__ __forceinline__ int chunks_of(int tokens) { return (tokens + kChunk - 1) / kChunk; }
+
 template <int DP>
-__global__ __launch_bounds__(256) void retention_chunk_kernel(
-    const float* __restrict__ p, int width, float* __restrict__ state, const int* __restrict__ read_rows,
-    const int* __restrict__ write_rows, const int* __restrict__ cu_q, const int* __restrict__ q_starts,
-    const float* __restrict__ decay, float* __restrict__ out, int heads, int dim, int vdim) {
+__global__ __launch_bounds__(256) void retention_local_kernel(const float* __restrict__ p, int width,
+                                                              const int* __restrict__ cu_q,
+                                                              const float* __restrict__ decay, float* __restrict__ out,
+                                                              float* __restrict__ local, int entries, int heads, int dim,
+                                                              int vdim, int vpad) {
   extern __shared__ float chunk_lds[];
   constexpr int LD = DP + 4;
-  constexpr int kPerRow = DP / 4;        // groups of 4 dims in a row
-  constexpr int kRowsAPass = 256 / kPerRow;
-  constexpr int kPasses = kChunk / kRowsAPass;
   float* const Qs = chunk_lds;                    // [64][LD]
   float* const Ks = Qs + kChunk * LD;             // [64][LD]
   float* const Vs = Ks + kChunk * LD;             // [64][16]
   float* const As = Vs + kChunk * 16;             // [4][16][kScoreLd]
-  float* const Ss = As + 4 * 16 * kScoreLd;       // [DP][16]
-  float* const pw = Ss + DP * 16;                 // [65]
+  float* const pw = As + 4 * 16 * kScoreLd;       // [65]
+  int entry = -1, left = blockIdx.x;
+  for (int e = 0; e < entries; ++e) {
+    const int have = chunks_of(cu_q[e + 1] - cu_q[e]);
+    if (left < have) {
+      entry = e;
+      break;
+    }
+    left -= have;
+  }
+  if (entry < 0) return;  // the grid is sized for the most chunks that the step's tokens could make
+  const int tb = cu_q[entry] + left * kChunk;
+  const int n = min(kChunk, cu_q[entry + 1] - tb);
+  const int h = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave;
+  const int w = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int r16 = lane % 16;
+  const int quad = lane / 16;
+  const float gamma = decay[h];
+  float* const As_w = As + w * 16 * kScoreLd;
+
+  if (tid <= kChunk) pw[tid] = powf(gamma, static_cast<float>(tid));  // g^0 = 1 also when g = 0
+  // loads are unconditional (a row past the end reads the chunk's last row, a dim past the head reads
+  // the head's last dim); what does not exist is cleared on its way to LDS
+  for (int idx = tid; idx < kChunk * (DP / 4); idx += 256) {
+    const int i = idx / (DP / 4);
+    const int d0 = 4 * (idx % (DP / 4));
+    const float* q = p + static_cast<int64_t>(tb + min(i, n - 1)) * width + static_cast<int64_t>(h) * dim;
+    const float* k = q + static_cast<int64_t>(heads) * dim;
+    float qv[4], kv[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int d = min(d0 + e, dim - 1);
+      qv[e] = q[d];
+      kv[e] = k[d];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const bool there = i < n && d0 + e < dim;
+      Qs[i * LD + d0 + e] = there ? qv[e] : 0.f;
+      Ks[i * LD + d0 + e] = there ? kv[e] : 0.f;
+    }
+  }
+  __syncthreads();
+
+  // scores of this wavefront's 16 queries against the key tiles up to the diagonal
+  f32x4v sc[4];
+#pragma unroll
+  for (int jt = 0; jt < 4; ++jt) sc[jt] = f32x4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+  for (int s = 0; s < DP / 4; ++s) {
+    const int d = 4 * s + quad;
+    const float a = Qs[(16 * w + r16) * LD + d];
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt)
+      if (jt <= w) sc[jt] = mfma_f32(a, Ks[(16 * jt + r16) * LD + d], sc[jt]);
+  }
+#pragma unroll
+  for (int jt = 0; jt < 4; ++jt) {
+    if (jt > w) continue;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int i = 16 * w + 4 * quad + e;  // query, key: local indices of the chunk
+      const int j = 16 * jt + r16;
+      As_w[(4 * quad + e) * kScoreLd + j] = j <= i ? sc[jt][e] * pw[i - j] : 0.f;
+    }
+  }
+  // the keys as the state takes them, k_j g^(n-1-j), in place (the scores are done with them)
+  __syncthreads();
+  for (int idx = tid; idx < kChunk * DP; idx += 256) {
+    const int j = idx / DP;
+    Ks[j * LD + idx % DP] *= j < n ? pw[n - 1 - j] : 0.f;
+  }
+  // the scores are made once; 16 value columns at a time go through them
+  for (int v0 = 0; v0 < vdim; v0 += 16) {
+    __syncthreads();  // the columns before are done with (and, the first time, the scores are whole)
+    for (int idx = tid; idx < kChunk * 16; idx += 256) {
+      const int i = idx / 16, c = idx % 16;
+      const float v = p[static_cast<int64_t>(tb + min(i, n - 1)) * width + 2ll * heads * dim + static_cast<int64_t>(h) * vdim +
+                        min(v0 + c, vdim - 1)];
+      Vs[idx] = (i < n && v0 + c < vdim) ? v : 0.f;
+    }
+    __syncthreads();
+    f32x4v o = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < 4 * (w + 1); ++s) {
+      const int j = 4 * s + quad;
+      o = mfma_f32(As_w[r16 * kScoreLd + j], Vs[j * 16 + r16], o);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int i = 16 * w + 4 * quad + e;
+      if (i < n && v0 + r16 < vdim)
+        out[static_cast<int64_t>(tb + i) * heads * vdim + static_cast<int64_t>(h) * vdim + v0 + r16] = o[e];
+    }
+    // what the chunk adds to the state: rows of tile dt, for every fourth tile
+    float* dst = local + ((static_cast<int64_t>(blockIdx.x) * heads + h) * DP) * vpad + v0;
+    for (int dt = w; dt < DP / 16; dt += 4) {
+      f32x4v up[2] = {f32x4v{0.f, 0.f, 0.f, 0.f}, f32x4v{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+      for (int s = 0; s < kChunk / 4; ++s) {
+        const int j = 4 * s + quad;
+        up[s % 2] = mfma_f32(Ks[j * LD + 16 * dt + r16], Vs[j * 16 + r16], up[s % 2]);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dst[static_cast<int64_t>(16 * dt + 4 * quad + e) * vpad + r16] = up[0][e] + up[1][e];
+    }
+  }
+}
+
+template <int DP>
+__global__ __launch_bounds__(256) void retention_carry_kernel(
+    const float* __restrict__ p, int width, float* __restrict__ state, const int* __restrict__ read_rows,
+    const int* __restrict__ write_rows, const int* __restrict__ cu_q, const int* __restrict__ q_starts,
+    const float* __restrict__ decay, float* __restrict__ out, const float* __restrict__ local, int heads, int dim,
+    int vdim, int vpad) {
+  __shared__ float Ss[DP * 16];
+  __shared__ float pw[kChunk + 1];
+  constexpr int kTiles = (DP / 16 + 3) / 4;  // state tiles of a wavefront
   const int entry = blockIdx.x;
   const int h = blockIdx.y;
   const int v0 = blockIdx.z * 16;
@@ -543,122 +664,85 @@ __global__ __launch_bounds__(256) void retention_chunk_kernel(
   const int t_end = cu_q[entry + 1];
   const float gamma = decay[h];
   const int64_t head_state = static_cast<int64_t>(dim) * vdim;
-  float* const As_w = As + w * 16 * kScoreLd;
-  const int64_t last = static_cast<int64_t>(t_end - 1);
+  int chunk = 0;  // number of this entry's first chunk
+  for (int e = 0; e < entry; ++e) chunk += chunks_of(cu_q[e + 1] - cu_q[e]);
 
-  // this thread's share of a chunk: 4 dims of `kPasses` rows of q and of k, 4 columns of one row of v;
-  // loads are unconditional (a row past the end reads the entry's last row, a dim past the head
-  // reads the head's last dim) and what does not exist is cleared when it goes to LDS
-  const int my_d = 4 * (tid % kPerRow);
-  const int my_row = tid / kPerRow;
-  const int v_row = tid / 4;
-  const int v_col = 4 * (tid % 4);
-  float qn[kPasses][4], kn[kPasses][4], vn[4];
-  auto fetch = [&](int tb) {
+  // this lane's operands of a chunk: its query row's dims 4 s + quad, and the 4 rows x 1 column of
+  // every state tile it moves on
+  float qa[DP / 4], qn[DP / 4], ua[kTiles][4], un[kTiles][4], oa[4], on[4];
+  auto fetch = [&](int tb, int number) {
 #pragma unroll
-    for (int u = 0; u < kPasses; ++u) {
-      const int64_t t = min(static_cast<int64_t>(tb + u * kRowsAPass + my_row), last);
-      const float* q = p + t * width + static_cast<int64_t>(h) * dim;
-      const float* k = q + static_cast<int64_t>(heads) * dim;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int d = min(my_d + e, dim - 1);
-        qn[u][e] = q[d];
-        kn[u][e] = k[d];
-      }
+    for (int e = 0; e < 4; ++e) {  // the chunk's own part of this lane's results
+      const int64_t t = min(tb + 16 * w + 4 * quad + e, t_end - 1);
+      on[e] = out[t * heads * vdim + static_cast<int64_t>(h) * vdim + min(v0 + r16, vdim - 1)];
     }
-    const float* v = p + min(static_cast<int64_t>(tb + v_row), last) * width + 2ll * heads * dim + static_cast<int64_t>(h) * vdim;
+    const int64_t t = min(tb + 16 * w + r16, t_end - 1);
+    const float* q = p + t * width + static_cast<int64_t>(h) * dim;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) vn[e] = v[min(v0 + v_col + e, vdim - 1)];
+    for (int s = 0; s < DP / 4; ++s) qn[s] = q[min(4 * s + quad, dim - 1)];
+    const float* src = local + ((static_cast<int64_t>(number) * heads + h) * DP) * vpad + v0 + r16;
+#pragma unroll
+    for (int u = 0; u < kTiles; ++u) {
+      const int dt = min(w + 4 * u, DP / 16 - 1);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) un[u][e] = src[static_cast<int64_t>(16 * dt + 4 * quad + e) * vpad];
+    }
   };
-  fetch(t_first);
+  fetch(t_first, chunk);
 
-  if (tid <= kChunk) pw[tid] = powf(gamma, static_cast<float>(tid));  // g^0 = 1 also when g = 0
+  if (tid <= kChunk) pw[tid] = powf(gamma, static_cast<float>(tid));
   const bool carried = q_starts[entry] > 0;
-  const float* src = state + (static_cast<int64_t>(read_rows[entry]) * heads + h) * head_state;
+  const float* from = state + (static_cast<int64_t>(read_rows[entry]) * heads + h) * head_state;
   for (int idx = tid; idx < DP * 16; idx += 256) {
     const int d = idx / 16, c = idx % 16;
-    Ss[idx] = (carried && d < dim && v0 + c < vdim) ? src[static_cast<int64_t>(d) * vdim + v0 + c] : 0.f;
+    Ss[idx] = (carried && d < dim && v0 + c < vdim) ? from[static_cast<int64_t>(d) * vdim + v0 + c] : 0.f;
   }
 
-  for (int tb = t_first; tb < t_end; tb += kChunk) {
+  for (int tb = t_first; tb < t_end; tb += kChunk, ++chunk) {
     const int n = min(kChunk, t_end - tb);
-    __syncthreads();  // the chunk before is done with; the state is whole
+    const int row = tb + 16 * w + r16;  // (as an operand; as a result the lane has rows 16 w + 4 quad + e)
 #pragma unroll
-    for (int u = 0; u < kPasses; ++u) {
-      const int i = u * kRowsAPass + my_row;
+    for (int s = 0; s < DP / 4; ++s) qa[s] = (row < t_end && 4 * s + quad < dim) ? qn[s] : 0.f;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const bool there = i < n && my_d + e < dim;
-        Qs[i * LD + my_d + e] = there ? qn[u][e] : 0.f;
-        Ks[i * LD + my_d + e] = there ? kn[u][e] : 0.f;
-      }
-    }
+    for (int u = 0; u < kTiles; ++u)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) Vs[v_row * 16 + v_col + e] = (v_row < n && v0 + v_col + e < vdim) ? vn[e] : 0.f;
-    __syncthreads();
-    if (tb + kChunk < t_end) fetch(tb + kChunk);  // on its way while this chunk is computed
-
-    // scores of this wavefront's 16 queries against the key tiles up to the diagonal, and the
-    // queries against the state; both read the same query operand
-    f32x4v sc[4], inter = {0.f, 0.f, 0.f, 0.f};
+      for (int e = 0; e < 4; ++e) ua[u][e] = un[u][e];
 #pragma unroll
-    for (int jt = 0; jt < 4; ++jt) sc[jt] = f32x4v{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 8
-    for (int s = 0; s < DP / 4; ++s) {
-      const int d = 4 * s + quad;
-      const float a = Qs[(16 * w + r16) * LD + d];
-      inter = mfma_f32(a, Ss[d * 16 + r16], inter);
+    for (int e = 0; e < 4; ++e) oa[e] = on[e];
+    if (tb + kChunk < t_end) fetch(tb + kChunk, chunk + 1);  // on its way while this chunk is computed
+    __syncthreads();  // the state is whole
+    // four sums side by side: a product waits for the one before it on the same sum
+    f32x4v part[4];
 #pragma unroll
-      for (int jt = 0; jt < 4; ++jt)
-        if (jt <= w) sc[jt] = mfma_f32(a, Ks[(16 * jt + r16) * LD + d], sc[jt]);
-    }
+    for (int u = 0; u < 4; ++u) part[u] = f32x4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int jt = 0; jt < 4; ++jt) {
-      if (jt > w) continue;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int i = 16 * w + 4 * quad + e;  // query, key: local indices of the chunk
-        const int j = 16 * jt + r16;
-        As_w[(4 * quad + e) * kScoreLd + j] = j <= i ? sc[jt][e] * pw[i - j] : 0.f;
-      }
-    }
-    __syncthreads();  // (a wavefront reads what its other lanes wrote)
-    f32x4v o = {0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < 4 * (w + 1); ++s) {
-      const int j = 4 * s + quad;
-      o = mfma_f32(As_w[r16 * kScoreLd + j], Vs[j * 16 + r16], o);
-    }
+    for (int s = 0; s < DP / 4; ++s) part[s % 4] = mfma_f32(qa[s], Ss[(4 * s + quad) * 16 + r16], part[s % 4]);
+    const f32x4v inter = (part[0] + part[1]) + (part[2] + part[3]);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int i = 16 * w + 4 * quad + e;
       if (i < n && v0 + r16 < vdim)
         out[static_cast<int64_t>(tb + i) * heads * vdim + static_cast<int64_t>(h) * vdim + v0 + r16] =
-            o[e] + pw[i + 1] * inter[e];
+            oa[e] + pw[i + 1] * inter[e];
     }
     __syncthreads();  // every wavefront has read the state
-
-    // the state behind the chunk: rows of tile dt, for every fourth tile
-    for (int dt = w; dt < DP / 16; dt += 4) {
-      f32x4v up = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int s = 0; s < kChunk / 4; ++s) {
-        const int j = 4 * s + quad;
-        const float kj = j < n ? Ks[j * LD + 16 * dt + r16] * pw[n - 1 - j] : 0.f;
-        up = mfma_f32(kj, Vs[j * 16 + r16], up);
-      }
+    for (int u = 0; u < kTiles; ++u) {
+      const int dt = w + 4 * u;
+      if (dt < DP / 16) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int d = 16 * dt + 4 * quad + e;
-        Ss[d * 16 + r16] = pw[n] * Ss[d * 16 + r16] + up[e];
+        for (int e = 0; e < 4; ++e) {
+          const int d = 16 * dt + 4 * quad + e;
+          Ss[d * 16 + r16] = pw[n] * Ss[d * 16 + r16] + ua[u][e];
+        }
       }
     }
   }
   __syncthreads();
-  float* dst = state + (static_cast<int64_t>(write_rows[entry]) * heads + h) * head_state;
+  float* to = state + (static_cast<int64_t>(write_rows[entry]) * heads + h) * head_state;
   for (int idx = tid; idx < DP * 16; idx += 256) {
     const int d = idx / 16, c = idx % 16;
-    if (d < dim && v0 + c < vdim) dst[static_cast<int64_t>(d) * vdim + v0 + c] = Ss[idx];
+    if (d < dim && v0 + c < vdim) to[static_cast<int64_t>(d) * vdim + v0 + c] = Ss[idx];
   }
 }
 
@@ -796,10 +880,18 @@ int mlr_heads_linear(const void* x, int64_t in_row, int in_stride, const void* w
   return 0;
 }
 
+// Floats of scratch memory that mlr_retention_scan needs for its chunked way (0: it will not go that way).
+int64_t mlr_retention_scratch(int total_tokens, int entries, int heads, int dim, int vdim) {
+  if (dim > 128 || total_tokens <= 0) return 0;
+  const int dp = dim <= 16 ? 16 : (dim <= 32 ? 32 : (dim <= 64 ? 64 : 128));
+  return static_cast<int64_t>(total_tokens / kChunk + entries) * heads * dp * ((vdim + 15) / 16 * 16);
+}
+
 int mlr_retention_scan(float* projected, int width, float* state, int state_rows, const int* read_rows,
                        const int* write_rows, const int* cu_q, const int* q_starts, const float* decay,
                        const float* cos, const float* sin, int rotary_dims, float key_scale, float* out, int entries,
-                       int heads, int dim, int vdim, int chunked, int total_tokens, hipStream_t stream) {
+                       int heads, int dim, int vdim, int chunked, int total_tokens, float* scratch, int64_t scratch_floats,
+                       hipStream_t stream) {
   MLR_REQUIRE(projected && state && read_rows && write_rows && cu_q && q_starts && decay && out, "null pointer");
   MLR_REQUIRE(entries > 0 && heads > 0 && dim > 0 && vdim > 0 && state_rows > 0, "sizes must be > 0");
   MLR_REQUIRE(dim <= 256, "a head's state has up to 256 rows");
@@ -810,10 +902,14 @@ int mlr_retention_scan(float* projected, int width, float* state, int state_rows
   MLR_REQUIRE(grid.y < 65536u && grid.z < 65536u, "too many heads or columns for one launch");
   if (chunked && dim <= 128) {  // wider heads keep the state of the token-by-token kernel
     const int dp = dim <= 16 ? 16 : (dim <= 32 ? 32 : (dim <= 64 ? 64 : 128));
-    const size_t lds = (2 * kChunk * (dp + 4) + kChunk * 16 + 4 * 16 * kScoreLd + dp * 16 + kChunk + 1) * sizeof(float);
+    const int vpad = static_cast<int>(grid.z) * 16;
+    const int max_chunks = total_tokens / kChunk + entries;  // sum over the entries of ceil(tokens / 64) is at most this
+    MLR_REQUIRE(total_tokens > 0 && scratch != nullptr, "the chunked kernels need the number of tokens and scratch memory");
+    MLR_REQUIRE(scratch_floats >= static_cast<int64_t>(max_chunks) * heads * dp * vpad, "the scratch memory is too small");
+    const size_t lds = (2 * kChunk * (dp + 4) + kChunk * 16 + 4 * 16 * kScoreLd + kChunk + 1) * sizeof(float);
     static bool configured = false;
     if (!configured) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(retention_chunk_kernel<128>),
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(retention_local_kernel<128>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
       if (e != hipSuccess) {
         set_error(std::string("mlr_retention_scan: cannot raise the LDS limit: ") + hipGetErrorString(e));
@@ -821,13 +917,16 @@ int mlr_retention_scan(float* projected, int width, float* state, int state_rows
       }
       configured = true;
     }
-    MLR_REQUIRE(total_tokens > 0, "the chunked kernel needs the number of tokens");
-    retention_rotate_kernel<<<total_tokens, 256, 0, stream>>>(const_cast<float*>(projected), width, cos, sin, rotary_dims,
-                                                              key_scale, heads, dim);
+    retention_rotate_kernel<<<total_tokens, 256, 0, stream>>>(projected, width, cos, sin, rotary_dims, key_scale, heads, dim);
     MLR_LAUNCH_CHECK();
+    const dim3 all(max_chunks, heads);
 #define MLR_CHUNK(DP)                                                                                              \
-  retention_chunk_kernel<DP><<<grid, 256, lds, stream>>>(projected, width, state, read_rows, write_rows, cu_q, q_starts, \
-                                                         decay, out, heads, dim, vdim)
+  do {                                                                                                             \
+    retention_local_kernel<DP><<<all, 256, lds, stream>>>(projected, width, cu_q, decay, out, scratch, entries, heads, dim, \
+                                                          vdim, vpad);                                             \
+    retention_carry_kernel<DP><<<grid, 256, 0, stream>>>(projected, width, state, read_rows, write_rows, cu_q, q_starts, \
+                                                         decay, out, scratch, heads, dim, vdim, vpad);             \
+  } while (0)
     if (dp == 16)
       MLR_CHUNK(16);
     else if (dp == 32)

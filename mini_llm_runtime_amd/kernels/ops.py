@@ -36,7 +36,10 @@ _SIGNATURES = {
         _I,
     ),
     "mlr_heads_linear": ([_VP, _I64, _I, _VP, _VP, _I64, _I, _VP, _I, _I, _I, _I, _I, _VP], _I),
-    "mlr_retention_scan": ([_VP, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _F, _VP, _I, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_retention_scan": (
+        [_VP, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _F, _VP, _I, _I, _I, _I, _I, _I, _VP, _I64, _VP], _I,
+    ),
+    "mlr_retention_scratch": ([_I, _I, _I, _I, _I], _I64),
     "mlr_retention_gate": ([_VP, _VP, _I, _I, _VP, _I, _I, _I, _I, _F, _VP], _I),
     "mlr_rmsnorm": ([_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _I, _F, _VP], _I),
     "mlr_add": ([_VP, _VP, _I, _I64, _VP], _I),
@@ -1150,11 +1153,16 @@ class HipOps:
             self._check(cos, "rotary cos", torch.float32, (tokens, rotary // 2))
             self._check(sin, "rotary sin", torch.float32, (tokens, rotary // 2))
         out = self._empty((tokens, heads * value_dim), torch.float32)
+        scratch, floats = None, 0
+        if chunked:
+            floats = int(self.lib.mlr_retention_scratch(tokens, entries, heads, head_dim, value_dim))
+            if floats:
+                scratch = self._empty((floats,), torch.float32)
         self._call(
             "mlr_retention_scan", self._ptr(projected), width, self._ptr(state), state.shape[0], self._ptr(read_rows),
             self._ptr(write_rows), self._ptr(ctx.cu_q), self._ptr(ctx.q_starts), self._ptr(decay), self._ptr(cos),
             self._ptr(sin), int(rotary), float(key_scale), self._ptr(out), entries, heads, head_dim, value_dim,
-            int(bool(chunked)), tokens, self._stream(),
+            int(bool(chunked)), tokens, self._ptr(scratch), floats, self._stream(),
         )
         return out
 
