@@ -501,14 +501,14 @@ __global__ __launch_bounds__(256) void retention_rotate_kernel(float* __restrict
 // q and k come rotated and scaled (retention_rotate_kernel).  Only S links the chunks, so the work is
 // cut in two.  retention_local_kernel: a workgroup per (chunk, head, 16 value columns), all chunks of
 // all entries at once, makes the chunk's own part of o (the sum over j) and its U.
-// retention_carry_kernel: a workgroup per (entry, head, 16 value columns) walks the entry's chunks in
-// order, adds g^(i+1) S^T q_i to o and moves S on by U: one small product and two barriers a chunk, its
-// operands asked for a chunk ahead.
-// Wavefront w of four owns the query rows 16 w .. 16 w + 15 of a chunk and every fourth 16-row tile of
-// the state.  LDS of the first kernel: the chunk's q and k [64][DP + 4] (DP: dim rounded up to 16, 32,
-// 64 or 128, zero padded; rows 4 words apart modulo 32 keep the operand reads of 16 rows x 4 columns
-// off each other's banks), its values [64][16], the masked scores per wavefront [16][68], the powers
-// g^0..g^64; of the second: the state [DP][16] and the powers.
+// retention_state_kernel walks every entry's chunks in order, element by element (S' = g^n S + U needs no
+// product), and leaves the state before every chunk; retention_apply_kernel, all chunks at once again, adds
+// g^(i+1) S^T q_i to o.  The chain from chunk to chunk is one multiply-add an element.
+// Wavefront w of four owns the query rows 16 w .. 16 w + 15 of a chunk and, in the first kernel, every
+// fourth 16-row tile of U.  LDS of the first kernel: the chunk's q and k [64][DP + 4] (DP: dim rounded up
+// to 16, 32, 64 or 128, zero padded; rows 4 words apart modulo 32 keep the operand reads of 16 rows x 4
+// columns off each other's banks), its values [64][16], the masked scores per wavefront [16][68], the
+// powers g^0..g^64.
 // Lane layouts of the product D[16x16] += A[16x4] B[4x16]: lane l holds A[l % 16][l / 16],
 // B[l / 16][l % 16] and D[4 (l / 16) + e][l % 16], e = 0..3.
 constexpr int kChunk = 64;
@@ -643,106 +643,114 @@ __global__ __launch_bounds__(256) void retention_local_kernel(const float* __res
   }
 }
 
-template <int DP>
-__global__ __launch_bounds__(256) void retention_carry_kernel(
-    const float* __restrict__ p, int width, float* __restrict__ state, const int* __restrict__ read_rows,
-    const int* __restrict__ write_rows, const int* __restrict__ cu_q, const int* __restrict__ q_starts,
-    const float* __restrict__ decay, float* __restrict__ out, const float* __restrict__ local, int heads, int dim,
-    int vdim, int vpad) {
-  __shared__ float Ss[DP * 16];
-  __shared__ float pw[kChunk + 1];
-  constexpr int kTiles = (DP / 16 + 3) / 4;  // state tiles of a wavefront
+// The state from chunk to chunk: S' = g^n S + U, element by element.  A thread owns one element of a head's
+// state and walks the entry's chunks; it leaves the state BEFORE every chunk where that chunk's U was
+// (`local`), for retention_apply_kernel.  The U values do not depend on the chain, so four chunks' loads are
+// on their way at a time.
+__global__ __launch_bounds__(256) void retention_state_kernel(float* __restrict__ state, const int* __restrict__ read_rows,
+                                                              const int* __restrict__ write_rows,
+                                                              const int* __restrict__ cu_q, const int* __restrict__ q_starts,
+                                                              const float* __restrict__ decay, float* __restrict__ local,
+                                                              int heads, int dim, int vdim, int dp, int vpad) {
   const int entry = blockIdx.x;
   const int h = blockIdx.y;
-  const int v0 = blockIdx.z * 16;
+  const int idx = blockIdx.z * 256 + threadIdx.x;
+  if (idx >= dp * vpad) return;
+  const int d = idx / vpad;
+  const int v = idx - d * vpad;
+  const bool real = d < dim && v < vdim;
+  const int tokens = cu_q[entry + 1] - cu_q[entry];
+  const int count = chunks_of(tokens);
+  int first = 0;  // number of this entry's first chunk
+  for (int e = 0; e < entry; ++e) first += chunks_of(cu_q[e + 1] - cu_q[e]);
+  const float gamma = decay[h];
+  const float whole = powf(gamma, static_cast<float>(kChunk));
+  const float rest = powf(gamma, static_cast<float>(tokens - (count - 1) * kChunk));  // the last chunk's tokens
+  const int64_t head_state = static_cast<int64_t>(dim) * vdim;
+  float s = 0.f;
+  if (real && q_starts[entry] > 0)
+    s = state[(static_cast<int64_t>(read_rows[entry]) * heads + h) * head_state + static_cast<int64_t>(d) * vdim + v];
+  float* u = local + ((static_cast<int64_t>(first) * heads + h) * dp) * vpad + idx;
+  const int64_t step = static_cast<int64_t>(heads) * dp * vpad;
+  for (int c0 = 0; c0 < count; c0 += 4) {
+    float add[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) add[k] = u[static_cast<int64_t>(min(c0 + k, count - 1)) * step];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int c = c0 + k;
+      if (c < count) {
+        u[static_cast<int64_t>(c) * step] = s;
+        s = (c == count - 1 ? rest : whole) * s + add[k];
+      }
+    }
+  }
+  if (real)
+    state[(static_cast<int64_t>(write_rows[entry]) * heads + h) * head_state + static_cast<int64_t>(d) * vdim + v] = s;
+}
+
+// o_i += g^(i+1) S^T q_i for every chunk at once, S the state before the chunk as retention_state_kernel
+// left it.  A workgroup per (chunk, head); wavefront w owns the query rows 16 w .. 16 w + 15, 16 value
+// columns at a time; the chunk's q goes through LDS, the state comes straight from memory.
+template <int DP>
+__global__ __launch_bounds__(256) void retention_apply_kernel(const float* __restrict__ p, int width,
+                                                              const int* __restrict__ cu_q,
+                                                              const int* __restrict__ q_starts,
+                                                              const float* __restrict__ decay, float* __restrict__ out,
+                                                              const float* __restrict__ local, int entries, int heads,
+                                                              int dim, int vdim, int vpad) {
+  constexpr int LD = DP + 4;
+  __shared__ float Qs[kChunk * LD];
+  int entry = -1, left = blockIdx.x;
+  for (int e = 0; e < entries; ++e) {
+    const int have = chunks_of(cu_q[e + 1] - cu_q[e]);
+    if (left < have) {
+      entry = e;
+      break;
+    }
+    left -= have;
+  }
+  if (entry < 0) return;  // the grid is sized for the most chunks that the step's tokens could make
+  if (left == 0 && q_starts[entry] == 0) return;  // the first chunk of a request: the state before it is zero
+  const int tb = cu_q[entry] + left * kChunk;
+  const int n = min(kChunk, cu_q[entry + 1] - tb);
+  const int h = blockIdx.y;
   const int tid = threadIdx.x;
   const int lane = tid % kWave;
   const int w = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int r16 = lane % 16;
   const int quad = lane / 16;
-  const int t_first = cu_q[entry];
-  const int t_end = cu_q[entry + 1];
   const float gamma = decay[h];
-  const int64_t head_state = static_cast<int64_t>(dim) * vdim;
-  int chunk = 0;  // number of this entry's first chunk
-  for (int e = 0; e < entry; ++e) chunk += chunks_of(cu_q[e + 1] - cu_q[e]);
-
-  // this lane's operands of a chunk: its query row's dims 4 s + quad, and the 4 rows x 1 column of
-  // every state tile it moves on
-  float qa[DP / 4], qn[DP / 4], ua[kTiles][4], un[kTiles][4], oa[4], on[4];
-  auto fetch = [&](int tb, int number) {
+  for (int idx = tid; idx < kChunk * (DP / 4); idx += 256) {
+    const int i = idx / (DP / 4);
+    const int d0 = 4 * (idx % (DP / 4));
+    const float* q = p + static_cast<int64_t>(tb + min(i, n - 1)) * width + static_cast<int64_t>(h) * dim;
+    float qv[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {  // the chunk's own part of this lane's results
-      const int64_t t = min(tb + 16 * w + 4 * quad + e, t_end - 1);
-      on[e] = out[t * heads * vdim + static_cast<int64_t>(h) * vdim + min(v0 + r16, vdim - 1)];
-    }
-    const int64_t t = min(tb + 16 * w + r16, t_end - 1);
-    const float* q = p + t * width + static_cast<int64_t>(h) * dim;
+    for (int e = 0; e < 4; ++e) qv[e] = q[min(d0 + e, dim - 1)];
 #pragma unroll
-    for (int s = 0; s < DP / 4; ++s) qn[s] = q[min(4 * s + quad, dim - 1)];
-    const float* src = local + ((static_cast<int64_t>(number) * heads + h) * DP) * vpad + v0 + r16;
-#pragma unroll
-    for (int u = 0; u < kTiles; ++u) {
-      const int dt = min(w + 4 * u, DP / 16 - 1);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) un[u][e] = src[static_cast<int64_t>(16 * dt + 4 * quad + e) * vpad];
-    }
-  };
-  fetch(t_first, chunk);
-
-  if (tid <= kChunk) pw[tid] = powf(gamma, static_cast<float>(tid));
-  const bool carried = q_starts[entry] > 0;
-  const float* from = state + (static_cast<int64_t>(read_rows[entry]) * heads + h) * head_state;
-  for (int idx = tid; idx < DP * 16; idx += 256) {
-    const int d = idx / 16, c = idx % 16;
-    Ss[idx] = (carried && d < dim && v0 + c < vdim) ? from[static_cast<int64_t>(d) * vdim + v0 + c] : 0.f;
+    for (int e = 0; e < 4; ++e) Qs[i * LD + d0 + e] = (i < n && d0 + e < dim) ? qv[e] : 0.f;
   }
-
-  for (int tb = t_first; tb < t_end; tb += kChunk, ++chunk) {
-    const int n = min(kChunk, t_end - tb);
-    const int row = tb + 16 * w + r16;  // (as an operand; as a result the lane has rows 16 w + 4 quad + e)
+  __syncthreads();
+  if (16 * w >= n) return;  // no query in this wavefront's rows
+  float power[4];
 #pragma unroll
-    for (int s = 0; s < DP / 4; ++s) qa[s] = (row < t_end && 4 * s + quad < dim) ? qn[s] : 0.f;
-#pragma unroll
-    for (int u = 0; u < kTiles; ++u)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) ua[u][e] = un[u][e];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) oa[e] = on[e];
-    if (tb + kChunk < t_end) fetch(tb + kChunk, chunk + 1);  // on its way while this chunk is computed
-    __syncthreads();  // the state is whole
-    // four sums side by side: a product waits for the one before it on the same sum
-    f32x4v part[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) part[u] = f32x4v{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < DP / 4; ++s) part[s % 4] = mfma_f32(qa[s], Ss[(4 * s + quad) * 16 + r16], part[s % 4]);
-    const f32x4v inter = (part[0] + part[1]) + (part[2] + part[3]);
+  for (int e = 0; e < 4; ++e) power[e] = powf(gamma, static_cast<float>(16 * w + 4 * quad + e + 1));
+  const float* sb = local + ((static_cast<int64_t>(blockIdx.x) * heads + h) * DP) * vpad;
+  for (int v0 = 0; v0 < vdim; v0 += 16) {
+    f32x4v part[2] = {f32x4v{0.f, 0.f, 0.f, 0.f}, f32x4v{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll 8
+    for (int s = 0; s < DP / 4; ++s)
+      part[s % 2] = mfma_f32(Qs[(16 * w + r16) * LD + 4 * s + quad], sb[static_cast<int64_t>(4 * s + quad) * vpad + v0 + r16],
+                             part[s % 2]);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int i = 16 * w + 4 * quad + e;
-      if (i < n && v0 + r16 < vdim)
-        out[static_cast<int64_t>(tb + i) * heads * vdim + static_cast<int64_t>(h) * vdim + v0 + r16] =
-            oa[e] + pw[i + 1] * inter[e];
-    }
-    __syncthreads();  // every wavefront has read the state
-#pragma unroll
-    for (int u = 0; u < kTiles; ++u) {
-      const int dt = w + 4 * u;
-      if (dt < DP / 16) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int d = 16 * dt + 4 * quad + e;
-          Ss[d * 16 + r16] = pw[n] * Ss[d * 16 + r16] + ua[u][e];
-        }
+      if (i < n && v0 + r16 < vdim) {
+        float* at = out + static_cast<int64_t>(tb + i) * heads * vdim + static_cast<int64_t>(h) * vdim + v0 + r16;
+        *at += power[e] * (part[0][e] + part[1][e]);
       }
     }
-  }
-  __syncthreads();
-  float* to = state + (static_cast<int64_t>(write_rows[entry]) * heads + h) * head_state;
-  for (int idx = tid; idx < DP * 16; idx += 256) {
-    const int d = idx / 16, c = idx % 16;
-    if (d < dim && v0 + c < vdim) to[static_cast<int64_t>(d) * vdim + v0 + c] = Ss[idx];
   }
 }
 
@@ -924,8 +932,10 @@ int mlr_retention_scan(float* projected, int width, float* state, int state_rows
   do {                                                                                                             \
     retention_local_kernel<DP><<<all, 256, lds, stream>>>(projected, width, cu_q, decay, out, scratch, entries, heads, dim, \
                                                           vdim, vpad);                                             \
-    retention_carry_kernel<DP><<<grid, 256, 0, stream>>>(projected, width, state, read_rows, write_rows, cu_q, q_starts, \
-                                                         decay, out, scratch, heads, dim, vdim, vpad);             \
+    retention_state_kernel<<<dim3(entries, heads, (DP * vpad + 255) / 256), 256, 0, stream>>>(                    \
+        state, read_rows, write_rows, cu_q, q_starts, decay, scratch, heads, dim, vdim, DP, vpad);                 \
+    retention_apply_kernel<DP><<<all, 256, 0, stream>>>(projected, width, cu_q, q_starts, decay, out, scratch, entries, \
+                                                        heads, dim, vdim, vpad);                                   \
   } while (0)
     if (dp == 16)
       MLR_CHUNK(16);
