@@ -77,7 +77,7 @@ int mlr_qkv_finish(const float* partial, int slices, const float* cos, const flo
 // pairing) is multiplied into the activated sums: y = act(x w^T + bias) * multiply.
 int mlr_gemm_simple(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
                     int out_is_f32, int swiglu, int dtype, int m, int n, int k, const void* multiply,
-                    float glu_limit, float glu_alpha, hipStream_t stream);
+                    const int* multiply_rows, float glu_limit, float glu_alpha, hipStream_t stream);
 
 // The same product in bfloat16 on the matrix cores (float32 accumulation).  Needs
 // k % 8 == 0 and 16-byte aligned x and w; any m and n.  With slices > 1 (a value
@@ -99,7 +99,7 @@ int mlr_gemm_bf16_kernel(int m, int n, int k, int slices);
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
                   int out_is_f32, int swiglu, int slices, int kernel, int m, int n, int k,
                   const float* row_sumsq, int sumsq_parts, float norm_eps, const void* multiply,
-                  float glu_limit, float glu_alpha, hipStream_t stream);
+                  const int* multiply_rows, float glu_limit, float glu_alpha, hipStream_t stream);
 
 // A product that finishes the residual stream (gemm_stream.hip): y = a w^T (+ bias), a [m, k] and w
 // [n, k] bfloat16; then, every workgroup for its own columns of all rows, stream[m, n] (float32, in

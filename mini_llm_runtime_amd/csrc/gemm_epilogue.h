@@ -31,6 +31,9 @@ struct GemmEpilogue {
   // g * sigmoid(glu_alpha * g) * (u + 1) with g = min(gate, glu_limit), u = clamp(up, -glu_limit, glu_limit).
   float glu_limit = 0.f;
   float glu_alpha = 0.f;
+  // int32 [M], or null: row m of the result takes row multiply_rows[m] of `multiply` (rows of a table
+  // gathered inside the epilogue, e.g. by token id) instead of row m.
+  const int* multiply_rows = nullptr;
 };
 
 constexpr int kEpNone = 0;
@@ -177,7 +180,8 @@ __device__ __forceinline__ void store4(const GemmEpilogue& ep, int64_t m, int n,
       }
     }
     if (ep.multiply != nullptr) {
-      const bf16* other = static_cast<const bf16*>(ep.multiply) + at;
+      const bf16* other = static_cast<const bf16*>(ep.multiply) +
+                          (ep.multiply_rows != nullptr ? static_cast<int64_t>(ep.multiply_rows[m]) * N + n : at);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         if (n + i < N) v[i] *= to_f32(other[i]);

@@ -1131,12 +1131,14 @@ int mlr_gemm_bf16_kernel(int m, int n, int k, int slices) { return choose_kernel
 // mlr_gemm_bf16_slices; not with swiglu) y is float32 [slices, m, n]: partial sums
 // over slices of k, the bias in slice 0, for the consumer to add up.
 // `swiglu` 2 and 3 are element-wise activations instead (squared ReLU, sigmoid; any n, after the
-// bias), and `multiply` (bfloat16 [m, n], or null) is multiplied into the activated sums.
+// bias), and `multiply` (bfloat16 [m, n], or null) is multiplied into the activated sums; with
+// `multiply_rows` (int32 [m]) row i takes row multiply_rows[i] of `multiply` (a table [rows, n]).
 // `swiglu` 5: rows (and bias) woven as for 1, y [m, n / 2] = g * sigmoid(glu_alpha g) * (u + 1) with
 // g = min(gate, glu_limit), u = clamp(up, -glu_limit, glu_limit).
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y, int out_is_f32,
                   int swiglu, int slices, int kernel, int m, int n, int k, const float* row_sumsq, int sumsq_parts,
-                  float norm_eps, const void* multiply, float glu_limit, float glu_alpha, hipStream_t stream) {
+                  float norm_eps, const void* multiply, const int* multiply_rows, float glu_limit, float glu_alpha,
+                  hipStream_t stream) {
   MLR_REQUIRE(x && w && y, "null pointer");
   MLR_REQUIRE(swiglu >= kEpNone && swiglu <= kEpClampedGlu, "unknown epilogue");
   MLR_REQUIRE(swiglu != kEpClampedGlu || (n % 4 == 0 && multiply == nullptr && glu_limit > 0.f),
@@ -1153,7 +1155,9 @@ int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f3
               "x and w must be 16-byte aligned");
   MLR_REQUIRE(row_sumsq == nullptr || (sumsq_parts > 0 && sumsq_parts <= (1 << 16) && norm_eps >= 0.f),
               "sums of squares come with their number per row (1..65536) and an eps >= 0");
-  GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu, row_sumsq, sumsq_parts, norm_eps, multiply, glu_limit, glu_alpha};
+  MLR_REQUIRE(multiply_rows == nullptr || multiply != nullptr, "row indices come with a multiplier");
+  GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu, row_sumsq, sumsq_parts, norm_eps, multiply, glu_limit, glu_alpha,
+                  multiply_rows};
   if (kernel == 0) kernel = choose_kernel(m, n, k, slices);
   // the 256 x 320 tile has no room for the activations and the multiplier in its epilogue
   if (kernel == 48 && (swiglu >= kEpRelu2 || multiply != nullptr)) kernel = 45;

@@ -19,7 +19,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                           const void* __restrict__ bias, int bias_is_f32,
                                                           void* __restrict__ y, int out_is_f32, int swiglu,
-                                                          const T* __restrict__ multiply, int M, int N, int K,
+                                                          const T* __restrict__ multiply,
+                                                          const int* __restrict__ multiply_rows, int M, int N, int K,
                                                           float glu_limit, float glu_alpha) {
   __shared__ float xs[kTK][kTM + 4];
   __shared__ float ws[kTK][kTN + 4];
@@ -120,7 +121,8 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
       } else if (swiglu == 4) {
         v = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
       }
-      if (multiply != nullptr) v *= to_f32(multiply[gm * N + gn]);
+      if (multiply != nullptr)
+        v *= to_f32(multiply[(multiply_rows != nullptr ? static_cast<int64_t>(multiply_rows[gm]) : gm) * N + gn]);
       if (out_is_f32)
         static_cast<float*>(y)[gm * N + gn] = v;
       else
@@ -135,7 +137,7 @@ using namespace mlr;
 
 extern "C" int mlr_gemm_simple(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
                                int out_is_f32, int swiglu, int dtype, int m, int n, int k, const void* multiply,
-                               float glu_limit, float glu_alpha, hipStream_t stream) {
+                               const int* multiply_rows, float glu_limit, float glu_alpha, hipStream_t stream) {
   MLR_REQUIRE(x && w && y, "null pointer");
   MLR_REQUIRE(m > 0 && n > 0 && k > 0, "sizes must be > 0");
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
@@ -151,12 +153,13 @@ extern "C" int mlr_gemm_simple(const void* x, const void* w, const void* bias, i
   if (dtype == kF32)
     gemm_simple_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(x),
                                                         static_cast<const float*>(w), bias, bias_is_f32, y,
-                                                        out_is_f32, swiglu, static_cast<const float*>(multiply), m, n, k,
-                                                        glu_limit, glu_alpha);
+                                                        out_is_f32, swiglu, static_cast<const float*>(multiply), multiply_rows,
+                                                        m, n, k, glu_limit, glu_alpha);
   else
     gemm_simple_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w),
                                                        bias, bias_is_f32, y, out_is_f32, swiglu,
-                                                       static_cast<const bf16*>(multiply), m, n, k, glu_limit, glu_alpha);
+                                                       static_cast<const bf16*>(multiply), multiply_rows, m, n, k, glu_limit,
+                                                       glu_alpha);
   MLR_LAUNCH_CHECK();
   return 0;
 }

@@ -49,8 +49,8 @@ _SIGNATURES = {
     "mlr_rope_table": ([_VP, _VP, _VP, _VP, _I, _I, _F, _VP], _I),
     "mlr_rope_kv_write": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_qkv_finish": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
-    "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP, _F, _F, _VP], _I),
-    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _I, _VP, _I, _F, _VP, _F, _F, _VP], _I),
+    "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP, _F, _F, _VP], _I),
+    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _I, _VP, _I, _F, _VP, _VP, _F, _F, _VP], _I),
     "mlr_moe_route": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _VP], _I),
     "mlr_moe_tile_rows": ([_I], _I),
     "mlr_moe_max_tiles": ([_I, _I, _I], _I),
@@ -478,6 +478,7 @@ class HipOps:
         activation: Optional[str] = None,
         multiply: Optional[torch.Tensor] = None,
         clamped_glu: Optional[tuple[float, float]] = None,
+        multiply_rows: Optional[torch.Tensor] = None,
     ) -> torch.Tensor:
         """x [M, K] times weight [N, K] transposed, plus bias [N]; F.linear semantics.
 
@@ -489,6 +490,8 @@ class HipOps:
         product's epilogue, in 32-bit, before the one rounding to the output's dtype.
         multiply: [M, N] in the engine's dtype; the (activated) sums are multiplied with it element
         by element before they are stored: a gate, sigmoid(x Wg^T) * other, in one kernel.
+        multiply_rows: int32 [M]; `multiply` is then a table [rows, N] of which result row i takes row
+        multiply_rows[i] (gathered inside the epilogue, e.g. by token id; the indices must lie inside the table).
 
         for_stream: the result is a part's output and goes nowhere but into the next norm as its
         delta (as with partial_sums); it may then come back unrun, as a `PendingLinear` that the norm
@@ -556,7 +559,12 @@ class HipOps:
         if out_dtype not in (torch.float32, self.dtype):
             raise KernelError(f"linear output must be float32 or {self.dtype}")
         bias_f32 = int(bias is not None and bias.dtype == torch.float32)
-        if multiply is not None:
+        if multiply_rows is not None:
+            if multiply is None:
+                raise KernelError("row indices come with a multiplier")
+            self._check(multiply_rows, "multiplier rows", torch.int32, (m,))
+            self._check(multiply, "multiplier table", self.dtype, (None, n))
+        elif multiply is not None:
             self._check(multiply, "multiplier", self.dtype, (m, n))
         if kernel == "auto" and self.dtype == torch.bfloat16 and k % 8 == 0:
             if slices is None:
@@ -573,15 +581,15 @@ class HipOps:
                 out_f32 = int(out_dtype == torch.float32)
             self._call(
                 "mlr_gemm_bf16", self._ptr(x), self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y), out_f32,
-                epilogue, slices, int(mfma_kernel), m, n, k, *scale, self._ptr(multiply), glu_limit, glu_alpha,
-                self._stream(),
+                epilogue, slices, int(mfma_kernel), m, n, k, *scale, self._ptr(multiply), self._ptr(multiply_rows),
+                glu_limit, glu_alpha, self._stream(),
             )
             return y
         y = self._empty((m, n // 2 if swiglu else n), out_dtype)
         self._call(
             "mlr_gemm_simple", self._ptr(x), self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y),
-            int(out_dtype == torch.float32), epilogue, self.code, m, n, k, self._ptr(multiply), glu_limit, glu_alpha,
-            self._stream(),
+            int(out_dtype == torch.float32), epilogue, self.code, m, n, k, self._ptr(multiply),
+            self._ptr(multiply_rows), glu_limit, glu_alpha, self._stream(),
         )
         return y
 

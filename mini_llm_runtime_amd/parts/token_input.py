@@ -25,7 +25,7 @@ class GatedTokenEmbedding(TokenInput):
         y = Wproj (gelu_tanh(Wgate x) * e[token]),   e: [vocab, dim], Wgate: [dim, H], Wproj: [H, dim].
 
     gelu_tanh(z) = 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))).  The gate product's epilogue
-    applies the activation and multiplies with the gathered rows.  The arrangement that holds this
+    applies the activation and multiplies with the token's row of the table, which it gathers itself.  The arrangement that holds this
     part norms y with `norm_weight` (a plain RMS weight) when it adds it to the stream.
     """
 
@@ -53,6 +53,7 @@ class GatedTokenEmbedding(TokenInput):
 
     def forward(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
         ops = ctx.ops
-        rows = ops.embedding(self.table, ctx.token_ids, out_dtype=ctx.dtype)
-        gated = ops.linear(x, self.gate_weight, None, activation="gelu_tanh", multiply=rows)
+        gated = ops.linear(
+            x, self.gate_weight, None, activation="gelu_tanh", multiply=self.table, multiply_rows=ctx.token_ids
+        )
         return ops.linear(gated, self.proj_weight, None, for_stream=True)

@@ -78,7 +78,7 @@ class TorchOps:
     # matrix products ---------------------------------------------------------------------
     def linear(
         self, x, weight, bias=None, out_dtype=None, kernel="auto", swiglu=False, partial_sums=False, for_stream=False,
-        activation=None, multiply=None, clamped_glu=None,
+        activation=None, multiply=None, clamped_glu=None, multiply_rows=None,
     ):
         self._count("linear")
         y = x.float() @ weight.float().t()
@@ -93,7 +93,7 @@ class TorchOps:
         elif activation is not None:
             raise ValueError(activation)
         if multiply is not None:
-            y = y * multiply.float()
+            y = y * (multiply.float() if multiply_rows is None else multiply[multiply_rows.long()].float())
         if clamped_glu is not None:  # rows woven like swiglu's, the bias with them
             limit, alpha = clamped_glu
             quads = y.view(y.shape[0], -1, 4)

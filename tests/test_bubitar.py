@@ -384,6 +384,9 @@ def test_gelu_product_with_gathered_rows(dtype, m, n, k):
     got = ops.linear(x.cuda(), w.cuda(), None, activation="gelu_tanh", multiply=rows)
     want = plain.gelu_tanh(x.double() @ w.double().T) * table[ids.long()].double()
     torch.testing.assert_close(got.double().cpu(), want, **_tolerance(dtype))
+    # the same with the rows gathered inside the product's epilogue
+    inside = ops.linear(x.cuda(), w.cuda(), None, activation="gelu_tanh", multiply=table.cuda(), multiply_rows=ids.cuda())
+    assert torch.equal(inside, got)
 
 
 @pytest.mark.parametrize("dtype", GPU_CASES)
