@@ -191,16 +191,16 @@ GPU_CASES = [
 
 def _compare(got, requests, weights, cfg, dtype, f32_bound=1e-4, row_bound=6e-2, together=2.5e-2):
     """float32: every value within 1e-4 of the logits' size.  bfloat16: all rows together within 2.5 %
-    (relative L2); every row within 6 %, but for a few (one in twenty) that may be off by up to 4 times what
-    rounding alone does to the worst row of their request (the plain implementation with its products
-    rounded to bfloat16).  A sublayer's output passes a norm before it is added, so where that output is
+    (relative L2); every row within 6 %, but for a few (one in twenty, and as many as rounding alone puts
+    beyond 6 %) that may be off by up to 4 times what rounding alone does to the worst row of their request
+    (the plain implementation with its products rounded to bfloat16).  A sublayer's output passes a norm before it is added, so where that output is
     near zero, or where a sink and one or two keys share the weight, every rounding moves the row by a
     percent, in the plain implementation as in the engine, and the worst row of hundreds is one where
     they all push the same way: the same rows stand out under every schedule.  A wrong key, page, slot or
     state changes a row by half and more, and most rows."""
     assert got, "no logits came back"
     num = den = 0.0
-    loose = rows = 0
+    loose = rows = loose_alone = 0
     for rid, toks in requests.items():
         ref = plain.forward(cfg, weights, toks)
         size = float(ref.pow(2).mean().sqrt())
@@ -208,6 +208,7 @@ def _compare(got, requests, weights, cfg, dtype, f32_bound=1e-4, row_bound=6e-2,
             with plain.rounded():
                 coarse = plain.forward(cfg, weights, toks)
             alone = (coarse - ref).pow(2).sum(-1).sqrt() / ref.pow(2).sum(-1).sqrt()
+            loose_alone += int((alone >= row_bound).sum())
         for pos in range(len(toks)):
             row = got[(rid, pos)].double()
             assert torch.isfinite(row).all(), f"{rid}:{pos} is not finite"
@@ -224,7 +225,8 @@ def _compare(got, requests, weights, cfg, dtype, f32_bound=1e-4, row_bound=6e-2,
             num += float(diff.pow(2).sum())
             den += float(ref[pos].pow(2).sum())
     if dtype != torch.float32:
-        assert loose <= 0.05 * rows + 1, f"{loose} of {rows} rows are ill-conditioned: the test's model is no yardstick"
+        # (as many as rounding alone puts beyond the bound, and a few)
+        assert loose <= 0.05 * rows + 1 + 1.5 * loose_alone, f"{loose} of {rows} rows are off by more than {row_bound}, {loose_alone} by rounding alone"
         assert (num / den) ** 0.5 < together, f"relative error of all rows {(num / den) ** 0.5:.3e}"
 
 
