@@ -874,7 +874,7 @@ DESIGN_VOCAB = 32768
 # The Bubitar decoder beside the Qwen2 decoder: the same width, query heads, head size, feed-forward width (both
 # feed-forwards have three matrices), layers and vocabulary.  Layers alternate retention (heads of dim x dim)
 # and latent attention (dim unrotated + 64 rotated query dimensions, a latent of 192: the cached row of 256 is
-# the widest the attention kernels take); every second latent layer reads the cache of the one before it.
+# the widest the matrix-core attention kernels take); every second latent layer reads the cache of the one before it.
 BUBITAR_POINTS = {
     # name: (width, heads, kv heads of the Qwen2 twin, head size, feed-forward width, layers run, token side dim)
     "hybrid-0.5b": (896, 14, 2, 64, 4864, 12, 64),

@@ -14,16 +14,16 @@
 
 namespace mlr {
 
-constexpr int kMaxHeadDim = 256;
+constexpr int kMaxHeadDim = 1024;  // the widest head (a cached latent row can be that wide); MAXD below is 256 or this
 
-template <typename T>
+template <typename T, int MAXD>
 __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ key_pages,
     const T* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ token_entry, const int* __restrict__ positions, T* __restrict__ out, int entries,
     int heads, int kv_heads, int head_dim, int block_size, int num_pages, float scale, int window, int chunk,
     const float* __restrict__ sinks) {
-  __shared__ float qs[kMaxHeadDim];
+  __shared__ float qs[MAXD];
   __shared__ float ps[kWave];
   __shared__ int64_t offs[kWave];
   __shared__ int64_t voffs[kWave];
@@ -48,7 +48,9 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
   const int first = first_visible_key(p, window, chunk);
   float m = -INFINITY;
   float l = 0.f;
-  float acc[kMaxHeadDim / kWave] = {0.f, 0.f, 0.f, 0.f};
+  float acc[MAXD / kWave];
+#pragma unroll
+  for (int j = 0; j < MAXD / kWave; ++j) acc[j] = 0.f;
   bool bad = false;
 
   for (int k0 = first; k0 <= p; k0 += kWave) {
@@ -83,13 +85,13 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     __syncthreads();
     const int count = min(kWave, p - k0 + 1);
 #pragma unroll
-    for (int j = 0; j < kMaxHeadDim / kWave; ++j) acc[j] *= alpha;
+    for (int j = 0; j < MAXD / kWave; ++j) acc[j] *= alpha;
     for (int i = 0; i < count; ++i) {
       if (offs[i] < 0) continue;
       const float pi = ps[i];
       const T* vp = value_pages + voffs[i];
 #pragma unroll
-      for (int j = 0; j < kMaxHeadDim / kWave; ++j) {
+      for (int j = 0; j < MAXD / kWave; ++j) {
         const int dim = lane + j * kWave;
         if (dim < head_dim) acc[j] = fmaf(pi, to_f32(vp[static_cast<int64_t>(dim) * block_size]), acc[j]);
       }
@@ -104,12 +106,12 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     const float alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
     l = l * alpha + expf(sink - m_new);
 #pragma unroll
-    for (int j = 0; j < kMaxHeadDim / kWave; ++j) acc[j] *= alpha;
+    for (int j = 0; j < MAXD / kWave; ++j) acc[j] *= alpha;
   }
   const bool any_bad = __any(bad);
   const float inv = 1.0f / l;
 #pragma unroll
-  for (int j = 0; j < kMaxHeadDim / kWave; ++j) {
+  for (int j = 0; j < MAXD / kWave; ++j) {
     const int dim = lane + j * kWave;
     if (dim < head_dim) orow[dim] = from_f32<T>(any_bad ? __builtin_nanf("") : acc[j] * inv);
   }
@@ -128,7 +130,7 @@ extern "C" int mlr_paged_attention_simple(const void* q, int64_t q_stride, const
   MLR_REQUIRE(q && key_pages && value_pages && block_table && token_entry && positions && out, "null pointer");
   MLR_REQUIRE(tokens > 0 && entries > 0 && heads > 0 && kv_heads > 0, "sizes must be > 0");
   MLR_REQUIRE(heads % kv_heads == 0, "query heads must be a multiple of KV heads");
-  MLR_REQUIRE(head_dim > 0 && head_dim <= kMaxHeadDim, "head_dim must be within 1..256");
+  MLR_REQUIRE(head_dim > 0 && head_dim <= kMaxHeadDim, "head_dim must be within 1..1024");
   MLR_REQUIRE(block_size > 0 && num_pages > 0 && table_width > 0, "page sizes must be > 0");
   MLR_REQUIRE(q_stride >= static_cast<int64_t>(heads) * head_dim, "q_stride is smaller than a row of queries");
   MLR_REQUIRE(scale > 0.f && scale < INFINITY, "scale must be positive and finite");
@@ -136,14 +138,27 @@ extern "C" int mlr_paged_attention_simple(const void* q, int64_t q_stride, const
   MLR_REQUIRE(heads < 65536, "too many heads for one launch");
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
   dim3 grid(tokens, heads);
+#define MLR_SIMPLE(T, MAXD)                                                                                      \
+  paged_attention_simple_kernel<T, MAXD><<<grid, kWave, 0, stream>>>(                                            \
+      static_cast<const T*>(q), q_stride, static_cast<const T*>(key_pages), static_cast<const T*>(value_pages),   \
+      block_table, table_width, token_entry, positions, static_cast<T*>(out), entries, heads, kv_heads, head_dim, \
+      block_size, num_pages, scale, window, chunk, sinks)
+  if (head_dim > 256) {
+    if (dtype == kF32)
+      MLR_SIMPLE(float, kMaxHeadDim);
+    else
+      MLR_SIMPLE(bf16, kMaxHeadDim);
+    MLR_LAUNCH_CHECK();
+    return 0;
+  }
   if (dtype == kF32)
-    paged_attention_simple_kernel<float><<<grid, kWave, 0, stream>>>(
+    paged_attention_simple_kernel<float, 256><<<grid, kWave, 0, stream>>>(
         static_cast<const float*>(q), q_stride, static_cast<const float*>(key_pages),
         static_cast<const float*>(value_pages), block_table, table_width, token_entry, positions,
         static_cast<float*>(out), entries, heads, kv_heads, head_dim, block_size, num_pages, scale, window, chunk,
         sinks);
   else
-    paged_attention_simple_kernel<bf16><<<grid, kWave, 0, stream>>>(
+    paged_attention_simple_kernel<bf16, 256><<<grid, kWave, 0, stream>>>(
         static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),
         static_cast<const bf16*>(value_pages), block_table, table_width, token_entry, positions,
         static_cast<bf16*>(out), entries, heads, kv_heads, head_dim, block_size, num_pages, scale, window, chunk,

@@ -14,10 +14,13 @@ from __future__ import annotations
 MAX_HEAD_DIM = 256  # the attention kernels keep a head's dims in the registers of one wavefront
 
 
-def check_attention_sizes(num_heads: int, num_kv_heads: int, head_dim: int) -> None:
+MAX_LATENT_ROW = 1024  # a cached latent row wider than MAX_HEAD_DIM runs the plain attention kernel, which takes this much
+
+
+def check_attention_sizes(num_heads: int, num_kv_heads: int, head_dim: int, limit: int = MAX_HEAD_DIM) -> None:
     """Raises ValueError for attention shapes no kernel of the library runs."""
-    if head_dim > MAX_HEAD_DIM:
+    if head_dim > limit:
         raise ValueError(
-            f"head_dim {head_dim}: the attention kernels take head sizes up to {MAX_HEAD_DIM} "
+            f"head_dim {head_dim}: the attention kernels take head sizes up to {limit} "
             f"({num_heads} query heads, {num_kv_heads} key/value heads asked for)"
         )

@@ -7,7 +7,7 @@ from typing import Optional
 import torch
 
 from ..cache.spec import PagedKVSpec
-from ..kernels.limits import check_attention_sizes
+from ..kernels.limits import MAX_LATENT_ROW, check_attention_sizes
 from .base import Mixer, Part, PositionEncoding
 from .context import MixerPlan, PlanInput, StepContext
 from .registry import build_part, register_part
@@ -72,7 +72,8 @@ class LatentAttention(Mixer):
         self.output_gate = bool(output_gate)
         # the one head size that the attention kernels and the pages see: a cached row [c ; r], padded
         self.kernel_dim = -(-(self.kv_rank + self.rot_dim) // 16) * 16
-        check_attention_sizes(num_heads, 1, self.kernel_dim)
+        # rows of up to 256 run on the matrix cores (in bfloat16); wider ones, up to 1,024, the plain kernel
+        check_attention_sizes(num_heads, 1, self.kernel_dim, limit=MAX_LATENT_ROW)
         self.position: Optional[PositionEncoding] = build_part("position", position) if position is not None else None
         if self.position is not None and getattr(self.position, "rotary_dim", self.rot_dim) > self.rot_dim:
             raise ValueError("the rotation covers more dimensions than the rotated part has")

@@ -96,12 +96,14 @@ CONFIGS = {
     ]),
     # one layer of each mixer and nothing else: what a mixer does is not blurred by the other
     "L": _model(128, 64, 1e-6, 4, [(_latent(2, 16, 16, 32, 32, 0.3, _rot(10000.0, 16, _YARN)), None)]),
+    # a cached row wider than the matrix-core attention kernels take (272 + 16 = 288): the plain kernel runs it
+    "W": _model(96, 64, 1e-6, 4, [(_latent(3, 16, 16, 24, 272, 0.2, _rot(10000.0, 16)), _ff(48, 1.5))]),
     "R": _model(128, 64, 1e-6, 4, [(_retention(2, 16, 32, (0.9, 0.995), _rot(10000.0, 8)), None)]),
 }
-BLOCK = {"A": 16, "B": 8, "C": 16, "D": 16, "L": 8, "R": 4}
+BLOCK = {"A": 16, "B": 8, "C": 16, "D": 16, "L": 8, "R": 4, "W": 16}
 LENGTHS = {
     "A": (1, 9, 50, 83, 37, 64), "B": (2, 19, 35, 66, 45), "C": (5, 17, 140, 70, 97), "D": (660, 341),
-    "L": (1, 24, 75, 41, 130), "R": (1, 24, 75, 41, 130),
+    "L": (1, 24, 75, 41, 130), "R": (1, 24, 75, 41, 130), "W": (3, 70, 41),
 }
 
 
