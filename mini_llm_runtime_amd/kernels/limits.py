@@ -14,6 +14,7 @@ from __future__ import annotations
 MAX_HEAD_DIM = 256  # the attention kernels keep a head's dims in the registers of one wavefront
 
 
+MAX_STATE_ROWS = 256  # the retention kernels keep a quarter of a head's state rows in a lane's registers
 MAX_LATENT_ROW = 1024  # a cached latent row wider than MAX_HEAD_DIM runs the plain attention kernel, which takes this much
 
 

@@ -7,6 +7,7 @@ from typing import Optional, Sequence
 import torch
 
 from ..cache.spec import SlotStateSpec
+from ..kernels.limits import MAX_STATE_ROWS
 from .base import Mixer, Part, PositionEncoding
 from .context import StepContext
 from .registry import build_part, register_part
@@ -43,6 +44,8 @@ class Retention(Mixer):
     ) -> None:
         if min(hidden_size, num_heads, head_dim, value_dim) <= 0:
             raise ValueError("Retention sizes must be > 0")
+        if head_dim > MAX_STATE_ROWS:  # refused here, not at the first step
+            raise ValueError(f"head_dim {head_dim}: the retention kernels take heads of up to {MAX_STATE_ROWS} dims")
         if len(decay) != num_heads or not all(0.0 <= float(g) <= 1.0 for g in decay):
             raise ValueError("Retention needs one decay within 0..1 per head")
         self.hidden_size = int(hidden_size)
